@@ -39,6 +39,7 @@ class RunNeed:
     cache_of: int                       # the run whose cache this run reads (itself: it owns one)
     cache: CacheNeed | None = None
     state: StateNeed | None = None
+    block_state: StateNeed | None = None    # what the layer's arrangement keeps per request besides its mixer
 
 
 @dataclass
@@ -122,6 +123,10 @@ class CacheManager:
                 area = torch.zeros((max_requests, *need.state.shape), dtype=need.state.dtype, device=device)
                 self.state_areas.append(area)
                 binding.state = area
+            if need.block_state is not None:
+                area = torch.zeros((max_requests, *need.block_state.shape), dtype=need.block_state.dtype, device=device)
+                self.state_areas.append(area)
+                binding.block_state = area
             self.bindings.append(binding)
 
     # ---- requests ------------------------------------------------------------------------

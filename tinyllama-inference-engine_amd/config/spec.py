@@ -50,6 +50,11 @@ class LayerSpec:
     # "layer_input" table), and its place
     layer_input: PartSpec | None = None
     layer_input_place: str = "side."
+    # something that stands between a norm and the sublayer that reads it (a part of the "sublayer_input" table, built
+    # once for the mixer and once for the feed-forward), and the places of the two
+    sublayer_input: PartSpec | None = None
+    mixer_input_place: str = "mixer_input."
+    feed_forward_input_place: str = "feed_forward_input."
 
 
 @dataclass(frozen=True)
@@ -68,6 +73,10 @@ class Run:
     # tell the passes apart.
     add_embedding: bool = False
     add_vector: tuple[str, int] | None = None
+    # What goes on after this run in place of its own result: a weighted sum over the embedding's output and the results
+    # of all runs so far, this one included (run i: i + 2 summands, in that order), with the weights of the tensor named
+    # here ([i + 2]).  A model uses this for all of its runs or for none.
+    depth_mix: str | None = None
 
 
 @dataclass(frozen=True)
@@ -106,6 +115,12 @@ class ModelSpec:
                 raise invalid_config(f"run {index} reads the cache of run {run.cache_of}, which does not run before it")
             if self.runs[run.cache_of].cache_of != run.cache_of:
                 raise invalid_config(f"run {index} reads the cache of run {run.cache_of}, which owns none")
+            if (run.depth_mix is None) != (self.runs[0].depth_mix is None):
+                raise invalid_config("either every run mixes the results so far into what goes on, or none does")
+            if run.depth_mix is not None:
+                shapes = [tensor.shape for tensor in self.shared_tensors if tensor.name == run.depth_mix]
+                if shapes != [(index + 2,)]:
+                    raise invalid_config(f"run {index} mixes the results so far with '{run.depth_mix}', which is no shared tensor [{index + 2}]")
             if run.add_vector is not None:
                 name, row = run.add_vector
                 shapes = [tensor.shape for tensor in self.shared_tensors if tensor.name == name]
@@ -115,8 +130,10 @@ class ModelSpec:
 
 @dataclass(frozen=True)
 class TensorSpec:
-    """A tensor a part expects in the checkpoint: its full name, shape and kind of values."""
+    """A tensor a part expects in the checkpoint: its full name, shape and kind of values.  An extent of -1 is a size
+    that the file gives and no configuration names (random weights draw `free_extent` there)."""
     name: str
     shape: tuple[int, ...]
-    init: str = "normal"        # how random weights draw it: "normal", "norm" (around 1), "offset" (a norm's weight stored around 0), "zeros", "forget_bias" (between 3 and 6)
+    init: str = "normal"        # how random weights draw it: "normal", "norm" (around 1), "offset" (a norm's weight stored around 0), "zeros", "forget_bias" (between 3 and 6), "fraction" (between 0 and 1), "mix" (weights of a sum: the last near 1, the others near 0)
+    free_extent: int = 16
     optional: bool = False       # absent is no error, present it is checked and not read (a tied head's matrix that some files still carry)

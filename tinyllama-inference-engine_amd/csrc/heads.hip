@@ -1,8 +1,8 @@
 // What stands between a mixer's per-head results and its output product when each head is normed by itself:
 //   o[t, h, :]   = a[t, h, :]                                            one result a head, or
 //                = a[t, first(h), :] - lambda * a[t, second(h), :]      two maps of attention a head, combined
-//   out[t, h, e] = o[e] / sqrt(mean(o^2) + eps) * weight[h * dv + e] * mult * sigmoid(gate[t, h * dv + e])
-// weight and gate are optional (null: 1).  Everything is float; `a` holds floats, the gate is read from a
+//   out[t, h, e] = o[e] / sqrt(mean(o^2) + eps) * weight[h * dv + e] * mult * f(gate[t, h * dv + e])
+// f is the sigmoid (gate_kind 0) or z * sigmoid(z) (gate_kind 1); weight and gate are optional (null: 1).  Everything is float; `a` holds floats, the gate is read from a
 // product's columns (any type, possibly partial sums), out is in the activation type.
 //
 // Two maps: `a` then holds 2 * heads results a token in the order in which the attention kernel wants its
@@ -18,7 +18,7 @@ template <typename D, typename W, typename A>
 __global__ void __launch_bounds__(256)
 head_combine_kernel(const float* __restrict__ a, int heads, int dv, int pair_group, int parts, float lambda, float eps,
                     const W* __restrict__ weight, float mult, const D* __restrict__ gate, int gate_nsplit,
-                    size_t gate_split_stride, int gate_row, int gate_col, A* __restrict__ out) {
+                    size_t gate_split_stride, int gate_row, int gate_col, int gate_kind, A* __restrict__ out) {
   const int t = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int h = blockIdx.y * 4 + wave;
   if (h >= heads) return;                              // (a whole wave; no barrier follows)
@@ -40,7 +40,7 @@ head_combine_kernel(const float* __restrict__ a, int heads, int dv, int pair_gro
     if (weight != nullptr) v *= to_float(weight[c]);
     if (gate != nullptr) {
       const float z = sum_splits(gate + static_cast<size_t>(t) * gate_row + gate_col + c, gate_nsplit, gate_split_stride);
-      v *= 1.f / (1.f + expf(-z));
+      v *= (gate_kind == 1 ? z : 1.f) / (1.f + expf(-z));
     }
     out[static_cast<size_t>(t) * heads * dv + c] = from_float<A>(v);
   };
@@ -79,10 +79,10 @@ using namespace tlie;
 // a product [nsplit][tokens][gate_row] of gate_dtype whose columns gate_col .. gate_col + heads * dv - 1 are read.
 extern "C" int tlie_head_combine(const float* a, int tokens, int heads, int dv, int pair_group, int parts, float lambda, float eps,
                                  const void* weight, int weight_dtype, float mult, const void* gate, int gate_dtype,
-                                 int gate_nsplit, long long gate_split_stride, int gate_row, int gate_col, void* out,
-                                 int out_dtype, void* stream) {
+                                 int gate_nsplit, long long gate_split_stride, int gate_row, int gate_col, int gate_kind,
+                                 void* out, int out_dtype, void* stream) {
   if (tokens <= 0 || heads <= 0 || dv <= 0 || pair_group < 0 || (pair_group > 0 && heads % pair_group != 0)) return kBadArgument;
-  if (parts < 1 || dv % parts != 0 || (parts > 1 && pair_group <= 0)) return kBadArgument;
+  if (parts < 1 || dv % parts != 0 || (parts > 1 && pair_group <= 0) || gate_kind < 0 || gate_kind > 1) return kBadArgument;
   if (gate != nullptr && (gate_nsplit < 1 || gate_col < 0 || gate_row < gate_col + heads * dv)) return kBadArgument;
   if (heads > 4 * 65535) return kBadArgument;
   const dim3 grid(tokens, (heads + 3) / 4);
@@ -91,7 +91,7 @@ extern "C" int tlie_head_combine(const float* a, int tokens, int heads, int dv, 
   if (gate_dtype == GC && weight_dtype == WC && out_dtype == AC) {                                                       \
     hipLaunchKernelGGL((head_combine_kernel<D, W, A>), grid, dim3(256), 0, s, a, heads, dv, pair_group, parts, lambda, eps,     \
                        (const W*)weight, mult, (const D*)gate, gate_nsplit, (size_t)gate_split_stride, gate_row, gate_col, \
-                       (A*)out);                                                                                          \
+                       gate_kind, (A*)out);                                                                                          \
     return launch_status();                                                                                              \
   }
   TLIE_CASE(kF32, float, kF32, float, kF32, float)

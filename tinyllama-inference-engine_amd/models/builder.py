@@ -58,6 +58,8 @@ class DecoderModel:
             if run.add_vector is not None and run.add_vector[0] not in self.run_vectors:
                 name = run.add_vector[0]
                 self.run_vectors[name] = keep_in(weights, weights[name].to(self.embedding.table.dtype).contiguous())
+            if run.depth_mix is not None and run.depth_mix not in self.run_vectors:
+                self.run_vectors[run.depth_mix] = keep_in(weights, weights[run.depth_mix].to(self.embedding.table.dtype).contiguous())
         release()
 
     @property
@@ -69,8 +71,10 @@ class DecoderModel:
     def run_needs(self) -> list[RunNeed]:
         needs = []
         for run in self.spec.runs:
-            mixer = self.blocks[run.layer].mixer
-            needs.append(RunNeed(cache_of=run.cache_of, cache=mixer.cache_need(), state=mixer.state_need()))
+            block = self.blocks[run.layer]
+            mixer = block.mixer
+            block_state = block.state_need() if hasattr(block, "state_need") else None
+            needs.append(RunNeed(cache_of=run.cache_of, cache=mixer.cache_need(), state=mixer.state_need(), block_state=block_state))
         return needs
 
     def forward(self, ctx, bindings) -> torch.Tensor:
@@ -84,6 +88,8 @@ class DecoderModel:
         as tensors there."""
         runs = self.spec.runs
         trace = getattr(ctx, "trace", None)
+        if runs[0].depth_mix is not None:
+            return self._forward_depth_mixed(ctx, bindings)
         few = ops.few_rows_route(ctx.num_tokens, self.dtype) and (trace is None or getattr(ctx, "trace_serving_route", False))
 
         def entry_norm(block):
@@ -125,6 +131,57 @@ class DecoderModel:
             trace["logits"] = logits.clone()
         return logits
 
+
+    def _forward_depth_mixed(self, ctx, bindings) -> torch.Tensor:
+        """A model whose runs hand on a weighted sum over the embedding's output and all results so far.  The results
+        are kept side by side for the length of the step, [runs + 2, tokens, hidden] floats: entry 0 the embedding's
+        output, entry i + 1 the residual that run i works on (it starts as what the run before handed on and ends as
+        the run's own result), the last entry what the last run hands on.  The norm that reads the residual next forms
+        the sum in its own kernel (it adds what the run's last sublayer left, mixes, writes the next run's residual
+        and norms it), so that a run costs no launch more than in a model without the mix."""
+        runs = self.spec.runs
+        trace = getattr(ctx, "trace", None)
+        first = self.embedding.forward(ctx.tokens, ctx)
+        tokens, hidden = first.shape
+        history = torch.empty((len(runs) + 2, tokens, hidden), dtype=torch.float32, device=first.device)
+        history[0].copy_(first)
+        history[1].copy_(first)
+        if trace is not None:
+            trace["embedding"] = first.float().clone()
+        normed = None
+        logits = None
+        for index, run in enumerate(runs):
+            if run.add_embedding or run.add_vector is not None:
+                raise ops.invalid_argument("runs that take the embedding or a vector again do not go with the mix over results")
+            block = self.blocks[run.layer]
+            if trace is not None:
+                ctx.trace_prefix = f"layer{index}."
+            kwargs = {"first_normed": normed} if normed is not None else {}
+            pending = block.forward(history[index + 1], None, ctx, bindings[index], **kwargs)
+            mix = dict(history=history, history_count=index + 2, history_weight=self.run_vectors[run.depth_mix])
+            last = index + 1 == len(runs)
+            next_norm = self.final_norm if last else self.blocks[runs[index + 1].layer].entry_norm()
+            if not hasattr(next_norm, "out_dtype"):
+                raise ops.invalid_argument("the mix over results is formed by the norm that follows it, which this norm cannot")
+            if last and trace is None:
+                if ctx.num_wanted == 0:
+                    # nothing is asked for: the state is up to date, the last sum has no reader
+                    return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)
+                rows = None if ctx.wants_all_rows else ctx.want_rows
+                normed = next_norm.add_forward(history[index + 1], pending, rows=rows, mixed=history[index + 2], **mix)
+            else:
+                normed = next_norm.add_forward(history[index + 1], pending, mixed=history[index + 2], **mix)
+                if trace is not None:
+                    trace[f"layer{index}.mixed"] = history[index + 2].clone()
+                    if last:
+                        if ctx.num_wanted == 0:
+                            return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)
+                        normed = normed if ctx.wants_all_rows else normed[ctx.want_rows.long()].contiguous()
+        logits = self.head.forward(normed)
+        if trace is not None:
+            trace["final_norm"] = normed.float().clone()
+            trace["logits"] = logits.clone()
+        return logits
 
     @staticmethod
     def _settle(residual, pending, dtype) -> None:

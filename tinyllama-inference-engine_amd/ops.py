@@ -104,6 +104,8 @@ def as_product(value) -> Product:
         return value
     if isinstance(value, torch.Tensor) and value.dim() == 2:
         return Product(value.contiguous(), 1)
+    if hasattr(value, "first_scale"):                     # a ScaledSum: added up here for whoever does not fuse it
+        return Product(value.dense(torch.float32).contiguous(), 1)
     raise invalid_argument("a part must return a [tokens, width] tensor or a Product")
 
 
@@ -570,11 +572,14 @@ def gated_recurrence(fused: Product, x_col: int, y_col: int, u: torch.Tensor, ga
     return out
 
 
+HEAD_GATES = {"sigmoid": 0, "silu": 1}      # what a head's gate becomes: sigmoid(z), or z * sigmoid(z)
+
+
 def head_combine(a: torch.Tensor, heads: int, value_dim: int, eps: float, out_dtype: torch.dtype, pair_group: int = 0,
                  pair_lambda: float = 0.0, weight: torch.Tensor | None = None, mult: float = 1.0,
-                 gate: Product | None = None, gate_col: int = 0, parts: int = 1) -> torch.Tensor:
+                 gate: Product | None = None, gate_col: int = 0, parts: int = 1, gate_kind: str = "sigmoid") -> torch.Tensor:
     """Each head's result normed by itself, on its way to the output product:
-    out[t, h, :] = o / sqrt(mean(o^2) + eps) * weight[h] * mult * sigmoid(gate[t, h]), with o = a[t, h] or, for two maps
+    out[t, h, :] = o / sqrt(mean(o^2) + eps) * weight[h] * mult * f(gate[t, h]) (f: `gate_kind`), with o = a[t, h] or, for two maps
     of attention a head (pair_group > 0: the query heads of one key head lie side by side in `a`, pair_group of them,
     first all first maps' key heads ... see the kernel), o = first - pair_lambda * second.  a: float32
     [tokens, heads (or 2 * heads) * value_dim]; weight (or None): [heads * value_dim]; gate (or None): a product whose
@@ -610,7 +615,7 @@ def head_combine(a: torch.Tensor, heads: int, value_dim: int, eps: float, out_dt
     _check(library().tlie_head_combine(_ptr(a), tokens, heads, value_dim, pair_group, int(parts), ctypes.c_float(pair_lambda),
                                        ctypes.c_float(eps), _ptr(weight), weight_code, ctypes.c_float(mult),
                                        _ptr(gate.data if gate is not None else None), gate_code, gate_nsplit,
-                                       ctypes.c_longlong(gate_stride), gate_row, gate_col, _ptr(out), dtype_code(out_dtype),
+                                       ctypes.c_longlong(gate_stride), gate_row, gate_col, HEAD_GATES[gate_kind], _ptr(out), dtype_code(out_dtype),
                                        _stream()), "head_combine")
     return out
 
@@ -666,6 +671,293 @@ def mlstm_scan(fused: Product, q_col: int, k_col: int, v_col: int, gates: torch.
                                      _ptr(values), _ptr(state), _ptr(seq_start), _ptr(seq_slot), _ptr(out), sequences, heads,
                                      dim, value_dim, ctypes.c_float(cap), ctypes.c_float(q_scale), slices, _ptr(parts),
                                      _stream()), "mlstm_scan")
+    return out
+
+
+@dataclass
+class ScaledSum:
+    """What a mixer of two branches hands on: first * first_scale + second * second_scale, not added up yet.  A norm
+    that knows it (`layer_norm`) adds both into the residual in its own kernel; anyone else asks for `dense()`."""
+    first: Product
+    first_scale: float
+    second: Product
+    second_scale: float
+
+    def dense(self, dtype: torch.dtype | None = None) -> torch.Tensor:
+        out = self.first.dense(torch.float32) * self.first_scale + self.second.dense(torch.float32) * self.second_scale
+        return out if dtype is None else out.to(dtype)
+
+
+def layer_norm(residual: torch.Tensor, delta, weight: torch.Tensor | None, bias: torch.Tensor | None, eps: float,
+               out_dtype: torch.dtype, rows: torch.Tensor | None = None, history: torch.Tensor | None = None,
+               history_count: int = 0, history_weight: torch.Tensor | None = None, mixed: torch.Tensor | None = None,
+               want_out: bool = True) -> torch.Tensor | None:
+    """residual += delta (a Product, a ScaledSum or None; all rows, in place), then out = (x - mean) / sqrt(var + eps)
+    * weight + bias of every row, means and variances float.  With `history` (float32 [entries, tokens, hidden] of which
+    the first history_count are read, the last of them being `residual` itself) what is normed is the weighted sum
+    sum_j history_weight[j] * history[j], which is also written to `mixed`.  With `rows` (int32 indices) only those
+    rows are normed and nothing but the result is written.  want_out False: only the sums."""
+    _device_tensor(residual, "residual", torch.float32)
+    if residual.dim() != 2:
+        raise invalid_shape("layer_norm: the residual is [tokens, hidden]")
+    tokens, hidden = residual.shape
+    if hidden > 16000:
+        raise invalid_argument("layer_norm: rows of at most 16000 values")
+    w_code = F32
+    if want_out:
+        _device_tensor(weight, "norm weight", (torch.float32, torch.bfloat16))
+        w_code = dtype_code(weight.dtype)
+        if weight.shape != (hidden,) or (bias is not None and (bias.shape != (hidden,) or bias.dtype != weight.dtype)):
+            raise invalid_shape("layer_norm: weight and bias need one entry per column, of one type")
+        if not eps > 0.0:
+            raise EngineError(ErrorCode.NUMERICAL, "a norm requires a positive epsilon")
+    parts = []
+    if isinstance(delta, ScaledSum):
+        parts = [(delta.first, delta.first_scale), (delta.second, delta.second_scale)]
+    elif delta is not None:
+        parts = [(as_product(delta), 1.0)]
+    for product, _ in parts:
+        _check_product(product, "delta")
+        if (product.rows, product.cols) != (tokens, hidden):
+            raise invalid_shape(f"layer_norm: delta [{product.rows}, {product.cols}] does not fit residual {list(residual.shape)}")
+    while len(parts) < 2:
+        parts.append((None, 0.0))
+    if history_count > 0:
+        _device_tensor(history, "history", torch.float32)
+        _device_tensor(history_weight, "history weight", (torch.float32, torch.bfloat16))
+        if want_out and history_weight.dtype != weight.dtype:
+            raise invalid_shape("layer_norm: the history's weights are of the norm's type")
+        w_code = dtype_code(history_weight.dtype)
+        if (history.dim() != 3 or tuple(history.shape[1:]) != (tokens, hidden) or history_count > history.shape[0]
+                or history_weight.shape != (history_count,)
+                or history[history_count - 1].data_ptr() != residual.data_ptr()):
+            raise invalid_shape("layer_norm: the history is [entries, tokens, hidden], its last entry read the residual itself")
+        if rows is None:
+            _device_tensor(mixed, "mixed", torch.float32)
+            if mixed.shape != residual.shape:
+                raise invalid_shape("layer_norm: the weighted sum has the residual's shape")
+    count = tokens
+    if rows is not None:
+        _device_tensor(rows, "rows", torch.int32)
+        count = rows.shape[0]
+    out = torch.empty((count, hidden), dtype=out_dtype, device=residual.device) if want_out else None
+    if count == 0 or tokens == 0:
+        return out
+
+    def code(product):
+        return dtype_code(product.data.dtype) if product is not None else F32
+    (d1, s1), (d2, s2) = parts
+    _check(library().tlie_layer_norm(
+        _ptr(residual), _ptr(d1.data if d1 is not None else None), code(d1), d1.nsplit if d1 is not None else 1,
+        ctypes.c_longlong(d1.split_stride if d1 is not None else 0), ctypes.c_float(s1),
+        _ptr(d2.data if d2 is not None else None), code(d2), d2.nsplit if d2 is not None else 1,
+        ctypes.c_longlong(d2.split_stride if d2 is not None else 0), ctypes.c_float(s2),
+        _ptr(history if history_count > 0 else None), ctypes.c_longlong(tokens * hidden), int(history_count),
+        _ptr(history_weight if history_count > 0 else None), _ptr(mixed if history_count > 0 and rows is None else None),
+        _ptr(weight if want_out else None), _ptr(bias if want_out else None), w_code, ctypes.c_float(eps if want_out else 1.0),
+        _ptr(out), dtype_code(out_dtype), _ptr(rows), count, hidden, _stream()), "layer_norm")
+    return out
+
+
+INPUT_CONV_MAX_TAPS = 8
+
+
+def input_conv(h: torch.Tensor, taps: torch.Tensor, state: torch.Tensor, ctx, out_dtype: torch.dtype) -> torch.Tensor:
+    """out = h + conv(h): a causal convolution per channel over each sequence's tokens of the step.  h: float32
+    [tokens, channels]; taps [channels, n], tap j weighs the input n - 1 - j tokens back; state: float32
+    [slots, max(n - 1, 1), channels] (the slots may lie apart: a part of a wider area), a request's last n - 1 inputs, oldest first, read for what came before the step and
+    brought up to the step's last token.  Rows of tokens whose slot is negative are left unwritten."""
+    _device_tensor(h, "h", torch.float32)
+    _device_tensor(taps, "taps", (torch.float32, torch.bfloat16))
+    if not isinstance(state, torch.Tensor) or not state.is_cuda or state.dtype != torch.float32:
+        raise invalid_argument("input_conv: the state is a float32 tensor on the GPU")
+    if h.dim() != 2 or taps.dim() != 2 or taps.shape[0] != h.shape[1] or not 1 <= taps.shape[1] <= INPUT_CONV_MAX_TAPS:
+        raise invalid_shape(f"input_conv: h {list(h.shape)} and taps {list(taps.shape)} do not fit (1 to {INPUT_CONV_MAX_TAPS} taps)")
+    tokens, channels = h.shape
+    count = taps.shape[1]
+    if state.dim() != 3 or tuple(state.shape[1:]) != (max(count - 1, 1), channels) or state.stride()[1:] != (channels, 1):
+        raise invalid_shape(f"input_conv: state {list(state.shape)} is not [slots, {max(count - 1, 1)}, {channels}] with rows side by side")
+    sequences = ctx.seq_slot.shape[0]
+    if ctx.token_seq.shape != (tokens,) or ctx.token_slot.shape != (tokens,) or ctx.seq_start.shape != (sequences + 1,):
+        raise invalid_shape("input_conv: the step's arrays do not fit the tokens")
+    out = torch.empty((tokens, channels), dtype=out_dtype, device=h.device)
+    if tokens == 0 or sequences == 0:
+        return out
+    _check(library().tlie_input_conv(_ptr(h), _ptr(taps), dtype_code(taps.dtype), _ptr(state), _ptr(ctx.token_seq),
+                                     _ptr(ctx.token_slot), _ptr(ctx.seq_start), _ptr(ctx.seq_slot), _ptr(out),
+                                     dtype_code(out_dtype), tokens, sequences, channels, count,
+                                     ctypes.c_longlong(state.stride(0)), _stream()), "input_conv")
+    return out
+
+
+def token_shift(x: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, ctx) -> torch.Tensor:
+    """out[m, t] = x_t + (x_(t-1) - x_t) * mu[m]: blends of a token's input with that of the token before it in its
+    sequence (zeros before the first).  x: [tokens, width] in the activation type; mu: [mixes, width]; state: float32
+    [slots, width], the last token's input of the step before, read and brought up to date.  Returns [mixes, tokens, width]."""
+    _device_tensor(x, "x", (torch.float32, torch.bfloat16))
+    _device_tensor(mu, "mu", (torch.float32, torch.bfloat16))
+    if not isinstance(state, torch.Tensor) or not state.is_cuda or state.dtype != torch.float32:
+        raise invalid_argument("token_shift: the state is a float32 tensor on the GPU")
+    if (x.dim() != 2 or mu.dim() != 2 or mu.shape[1] != x.shape[1] or state.dim() != 2 or state.shape[1] != x.shape[1]
+            or state.stride(1) != 1):
+        raise invalid_shape("token_shift: x [tokens, width], mu [mixes, width], state [slots, width] (the slots may lie apart)")
+    tokens, width = x.shape
+    sequences = ctx.seq_slot.shape[0]
+    if ctx.token_seq.shape != (tokens,) or ctx.token_slot.shape != (tokens,) or ctx.seq_start.shape != (sequences + 1,):
+        raise invalid_shape("token_shift: the step's arrays do not fit the tokens")
+    out = torch.empty((mu.shape[0], tokens, width), dtype=x.dtype, device=x.device)
+    if tokens == 0 or sequences == 0:
+        return out
+    _check(library().tlie_token_shift(_ptr(x), dtype_code(x.dtype), _ptr(mu), dtype_code(mu.dtype), _ptr(state),
+                                      _ptr(ctx.token_seq), _ptr(ctx.token_slot), _ptr(ctx.seq_start), _ptr(ctx.seq_slot),
+                                      _ptr(out), tokens, sequences, width, mu.shape[0], ctypes.c_longlong(state.stride(0)),
+                                      _stream()), "token_shift")
+    return out
+
+
+def xielu(pre: Product, numbers: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """softplus(p) z^2 + z / 2 for z > 0, (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2 otherwise, (p, q) = numbers."""
+    _check_product(pre, "pre")
+    _device_tensor(numbers, "numbers", (torch.float32, torch.bfloat16))
+    if numbers.shape != (2,):
+        raise invalid_shape("xielu: two numbers")
+    out = torch.empty((pre.rows, pre.cols), dtype=out_dtype, device=pre.data.device)
+    if out.numel() == 0:
+        return out
+    _check(library().tlie_xielu(_ptr(pre.data), dtype_code(pre.data.dtype), pre.nsplit, ctypes.c_longlong(pre.split_stride),
+                                _ptr(numbers), dtype_code(numbers.dtype), _ptr(out), dtype_code(out_dtype),
+                                ctypes.c_longlong(pre.rows * pre.cols), _stream()), "xielu")
+    return out
+
+
+def rotate_heads(fused: Product, col: int, positions: torch.Tensor, inv_freq: torch.Tensor | None, rot_dim: int, heads: int,
+                 heads_a: int, dim: int, scale_a: float, scale_b: float, tail: int = 0) -> torch.Tensor:
+    """Columns col .. of a product as floats on their way into a scan: `heads` heads of `dim` whose first rot_dim dims
+    turn by the token's position (dim i with dim i + rot_dim / 2, angle position * inv_freq[i]), the first heads_a of
+    them times scale_a afterwards and the others times scale_b, and `tail` more columns as they are."""
+    _check_product(fused, "fused")
+    _device_tensor(positions, "positions", torch.int32)
+    if rot_dim > 0:
+        _device_tensor(inv_freq, "inv_freq", torch.float32)
+        if inv_freq.shape != (rot_dim // 2,):
+            raise invalid_shape("rotate_heads: one frequency a pair")
+    if (rot_dim < 0 or rot_dim % 2 or rot_dim > dim or col < 0 or tail < 0 or col + heads * dim + tail > fused.cols
+            or positions.shape != (fused.rows,)):
+        raise invalid_shape("rotate_heads: the heads do not lie in the product's columns")
+    out = torch.empty((fused.rows, heads * dim + tail), dtype=torch.float32, device=fused.data.device)
+    if fused.rows == 0:
+        return out
+    _check(library().tlie_rotate_heads(_ptr(fused.data), dtype_code(fused.data.dtype), fused.nsplit,
+                                       ctypes.c_longlong(fused.split_stride), fused.cols, int(col), _ptr(positions),
+                                       _ptr(inv_freq if rot_dim > 0 else None), int(rot_dim), heads, heads_a, dim,
+                                       ctypes.c_float(scale_a), ctypes.c_float(scale_b), int(tail), _ptr(out), fused.rows,
+                                       _stream()), "rotate_heads")
+    return out
+
+
+LOW_RANK_DECAYS = {"sigmoid_root": 0, "exp_neg_exp": 1}
+
+
+def low_rank_decay(low: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, kind: str, tau: float = 1.0,
+                   inner_tanh: bool = False) -> torch.Tensor:
+    """Decays per token and channel from a low-rank product: z = bias + weight . f(low) (f: tanh or the identity), then
+    "sigmoid_root": sigmoid(z)^(1 / tau); "exp_neg_exp": exp(-exp(z)).  low: float32 [tokens, rank]; weight [channels, rank].
+    Float throughout; returns float32 [tokens, channels]."""
+    _device_tensor(low, "low", torch.float32)
+    _device_tensor(weight, "weight", (torch.float32, torch.bfloat16))
+    if low.dim() != 2 or weight.dim() != 2 or weight.shape[1] != low.shape[1] or low.shape[1] > 4096:
+        raise invalid_shape("low_rank_decay: low [tokens, rank], weight [channels, rank], rank up to 4096")
+    if bias is not None:
+        _device_tensor(bias, "bias", weight.dtype)
+        if bias.shape != (weight.shape[0],):
+            raise invalid_shape("low_rank_decay: one bias a channel")
+    if kind not in LOW_RANK_DECAYS or (kind == "sigmoid_root" and not tau > 0.0):
+        raise invalid_argument("low_rank_decay: an unknown kind, or a root that is not positive")
+    out = torch.empty((low.shape[0], weight.shape[0]), dtype=torch.float32, device=low.device)
+    if low.shape[0] == 0:
+        return out
+    _check(library().tlie_low_rank_decay(_ptr(low), int(inner_tanh), _ptr(weight), _ptr(bias), dtype_code(weight.dtype),
+                                         LOW_RANK_DECAYS[kind], ctypes.c_float(tau), _ptr(out), low.shape[0], weight.shape[0],
+                                         low.shape[1], _stream()), "low_rank_decay")
+    return out
+
+
+SCAN_MAX_DIM = 256             # the largest query/key size of a head that the scan keeps in registers
+SCAN_SLICE = 32                # tokens of a slice of the sliced walk (the kernel's kScanSlice)
+SCAN_SLICED_FROM = 96          # tokens a sequence brings from which the sliced walk pays
+
+
+def decay_scan_state_shape(heads: int, dim: int, value_dim: int) -> tuple[int, ...]:
+    """A request's state row for `decay_scan`: per head and tile of 64 value columns, S as [dim][64]."""
+    return (heads, (value_dim + 63) // 64, dim * 64)
+
+
+def decay_scan(q: tuple[Product, int], k: tuple[Product, int], v: tuple[Product, int], state: torch.Tensor, seq_start: torch.Tensor,
+               seq_slot: torch.Tensor, heads: int, dim: int, value_dim: int, decay: torch.Tensor | None = None,
+               head_decay: torch.Tensor | None = None, bonus: torch.Tensor | None = None, q_scale: float = 1.0,
+               k_scale: float = 1.0, max_new: int = 1) -> torch.Tensor:
+    """Linear attention with a decaying matrix state over the step's tokens, sequence by sequence (see
+    csrc/decay_scan.hip): S' = diag(w) S + k v^T, o = S'^T q per head; with `bonus` (float32 [heads * dim]) the result is
+    read before the token joins the state, o = (S + diag(bonus) k v^T)^T q.  q, k, v: (product, first column), of one
+    type; the decays w either `head_decay` (float32 [heads], one a head) or `decay` (float32 [tokens, heads * dim], one a
+    token and key channel).  Carries `state` (float32 [slots, *decay_scan_state_shape]) for sequences whose slot is not
+    negative (or [slots, floats] rows that begin with that shape's floats); returns float32 [tokens, heads * value_dim].  max_new: the most tokens any sequence brings in this step;
+    from SCAN_SLICED_FROM on the tokens are taken in slices of SCAN_SLICE that run side by side."""
+    for name, (product, _) in (("q", q), ("k", k), ("v", v)):
+        _check_product(product, name)
+    _device_tensor(state, "state", torch.float32)
+    _device_tensor(seq_start, "seq_start", torch.int32)
+    _device_tensor(seq_slot, "seq_slot", torch.int32)
+    tokens = q[0].rows
+    code = dtype_code(q[0].data.dtype)
+    if k[0].rows != tokens or v[0].rows != tokens or dtype_code(k[0].data.dtype) != code or dtype_code(v[0].data.dtype) != code:
+        raise invalid_shape("decay_scan: q, k and v have one row a token and one type")
+    if not 0 < dim <= SCAN_MAX_DIM or heads <= 0 or value_dim <= 0:
+        raise invalid_argument(f"decay_scan: heads of 1 to {SCAN_MAX_DIM} query dims")
+    shape = decay_scan_state_shape(heads, dim, value_dim)
+    if state.dim() == 2:                # a row that holds more than the scan's part, which comes first
+        if state.shape[1] < shape[0] * shape[1] * shape[2]:
+            raise invalid_shape(f"decay_scan: state rows of {state.shape[1]} floats do not hold {shape}")
+    elif state.dim() != 4 or tuple(state.shape[1:]) != shape:
+        raise invalid_shape(f"decay_scan: state {list(state.shape)} is not [slots, {shape}]")
+    sequences = seq_slot.shape[0]
+    if seq_start.shape != (sequences + 1,):
+        raise invalid_shape("decay_scan: seq_start needs one entry more than there are sequences")
+    for (product, col), size in ((q, heads * dim), (k, heads * dim), (v, heads * value_dim)):
+        if col < 0 or col + size > product.cols:
+            raise invalid_shape("decay_scan: q, k or v do not lie in their product's columns")
+    if (decay is None) == (head_decay is None):
+        raise invalid_argument("decay_scan: decays come either one a head or one a token and channel")
+    kind = 0
+    if decay is not None:
+        _device_tensor(decay, "decay", torch.float32)
+        if decay.shape != (tokens, heads * dim):
+            raise invalid_shape("decay_scan: one decay a token and key channel")
+        kind = 1
+    else:
+        _device_tensor(head_decay, "head_decay", torch.float32)
+        if head_decay.shape != (heads,):
+            raise invalid_shape("decay_scan: one decay a head")
+    if bonus is not None:
+        _device_tensor(bonus, "bonus", torch.float32)
+        if kind != 1 or bonus.shape != (heads * dim,):
+            raise invalid_shape("decay_scan: a bonus goes with decays per channel and has one entry a key channel")
+        kind = 2
+    out = torch.empty((tokens, heads * value_dim), dtype=torch.float32, device=state.device)
+    if tokens == 0 or sequences == 0:
+        return out
+    slices, parts = 0, None
+    if max_new >= SCAN_SLICED_FROM:
+        slices = (min(int(max_new), tokens) + SCAN_SLICE - 1) // SCAN_SLICE
+        parts = torch.empty((sequences, slices, shape[0], shape[1], shape[2] + dim), dtype=torch.float32, device=state.device)
+
+    def columns(pair):
+        product, col = pair
+        return (_ptr(product.data), product.nsplit, ctypes.c_longlong(product.split_stride), product.cols, int(col))
+    _check(library().tlie_decay_scan(*columns(q), *columns(k), *columns(v), code, kind, _ptr(decay), _ptr(head_decay), _ptr(bonus),
+                                     ctypes.c_float(q_scale), ctypes.c_float(k_scale), _ptr(state), _ptr(seq_start),
+                                     _ptr(seq_slot), _ptr(out), sequences, heads, dim, value_dim, slices, _ptr(parts),
+                                     ctypes.c_longlong(state.stride(0)), _stream()), "decay_scan")
     return out
 
 

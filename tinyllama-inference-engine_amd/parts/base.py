@@ -67,6 +67,7 @@ class Binding:
     cache: torch.Tensor | None = None   # [pages, *need.page_shape(page_size)] of the run whose cache is read
     writes: bool = True                 # this run owns the cache and writes the step's keys and values
     state: torch.Tensor | None = None   # [request slots, *shape] for a mixer with state of its own
+    block_state: torch.Tensor | None = None   # [request slots, *shape] for what the layer's arrangement keeps itself
 
 
 class Part:

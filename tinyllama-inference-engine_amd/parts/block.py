@@ -19,15 +19,48 @@ from .base import ResidualTarget
 
 @register("block", "pre_norm")
 class PreNormBlock:
+    """x += mixer(norm(x)), then, if the layer has a feed-forward, x += feed_forward(norm(x)).  With
+    `LayerSpec.sublayer_input` a part of the "sublayer_input" table stands between each norm and its sublayer (built
+    once for each); what such parts keep per request is this block's state, one row of it each."""
+
     def __init__(self, layer: LayerSpec, dtype, device):
+        from ..config.spec import PartSpec
+        from ..errors import invalid_config
         self.layer = layer
         self.dtype = dtype
-        self.mixer_norm = lookup("norm", layer.mixer_norm.kind)(layer.mixer_norm, dtype, device)
-        self.mixer = lookup("mixer", layer.mixer.kind)(layer.mixer, dtype, device)
-        self.feed_forward_norm = lookup("norm", layer.feed_forward_norm.kind)(layer.feed_forward_norm, dtype, device)
-        self.feed_forward = lookup("feed_forward", layer.feed_forward.kind)(layer.feed_forward, dtype, device)
+        between = layer.sublayer_input
 
-    _PARTS = ("mixer_norm", "mixer", "feed_forward_norm", "feed_forward")
+        def norm(spec):
+            if between is not None:         # what stands behind the norm reads floats
+                spec = PartSpec(spec.kind, {**dict(spec.params), "out": "float32"})
+            built = lookup("norm", spec.kind)(spec, dtype, device)
+            if between is not None and getattr(built, "out_dtype", None) != torch.float32:
+                raise invalid_config(f"a norm '{spec.kind}' cannot leave floats for what stands between it and its sublayer")
+            return built
+        self.mixer_norm = norm(layer.mixer_norm)
+        self.mixer = lookup("mixer", layer.mixer.kind)(layer.mixer, dtype, device)
+        self.feed_forward_norm = self.feed_forward = self.mixer_input = self.feed_forward_input = None
+        if layer.feed_forward is not None:
+            self.feed_forward_norm = norm(layer.feed_forward_norm)
+            self.feed_forward = lookup("feed_forward", layer.feed_forward.kind)(layer.feed_forward, dtype, device)
+        if between is not None:
+            self.mixer_input = lookup("sublayer_input", between.kind)(between, dtype, device)
+            if self.feed_forward is not None:
+                self.feed_forward_input = lookup("sublayer_input", between.kind)(between, dtype, device)
+        # the route on which norms are folded into products and products add into the residual is for the plain layer
+        self.plain = between is None and self.feed_forward is not None
+
+    @classmethod
+    def _parts(cls, layer: LayerSpec):
+        """(attribute, registry table, the layer's spec of it) of the parts this layer has."""
+        parts = [("mixer_norm", "norm", layer.mixer_norm), ("mixer", "mixer", layer.mixer)]
+        if layer.sublayer_input is not None:
+            parts.append(("mixer_input", "sublayer_input", layer.sublayer_input))
+        if layer.feed_forward is not None:
+            parts += [("feed_forward_norm", "norm", layer.feed_forward_norm), ("feed_forward", "feed_forward", layer.feed_forward)]
+            if layer.sublayer_input is not None:
+                parts.append(("feed_forward_input", "sublayer_input", layer.sublayer_input))
+        return parts
 
     @staticmethod
     def _place(layer: LayerSpec, attribute: str) -> str:
@@ -37,15 +70,21 @@ class PreNormBlock:
     @classmethod
     def tensor_specs(cls, layer: LayerSpec):
         specs = []
-        for attribute in cls._PARTS:
-            part_spec = getattr(layer, attribute)
-            table = {"mixer_norm": "norm", "feed_forward_norm": "norm"}.get(attribute, attribute)
+        for attribute, table, part_spec in cls._parts(layer):
             specs += lookup(table, part_spec.kind).tensor_specs(part_spec, cls._place(layer, attribute))
         return specs
 
     def load(self, weights):
-        for attribute in self._PARTS:
+        for attribute, _, _ in self._parts(self.layer):
             getattr(self, attribute).load(weights, self._place(self.layer, attribute))
+
+    def state_need(self):
+        """What the parts between norms and sublayers keep per request: a row each, [parts, rows, channels]."""
+        from .base import StateNeed
+        inputs = [part for part in (self.mixer_input, self.feed_forward_input) if part is not None]
+        if not inputs:
+            return None
+        return StateNeed((len(inputs), *inputs[0].state_shape()), torch.float32)
 
     def entry_norm(self):
         """The norm that reads the residual first in this block: whoever writes the residual before
@@ -54,12 +93,12 @@ class PreNormBlock:
 
     @property
     def graph_safe(self) -> bool:
-        return all(getattr(part, "graph_safe", False)
-                   for part in (self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward))
+        return all(getattr(getattr(self, attribute), "graph_safe", False) for attribute, _, _ in self._parts(self.layer))
 
-    def forward(self, residual, pending, ctx, binding, next_norm=None):
+    def forward(self, residual, pending, ctx, binding, next_norm=None, first_normed=None):
         """`pending`: what the residual still lacks (a product, a `ResidualUpdated`, or None).
         `next_norm`: the norm that reads the residual after this block, if the caller knows it.
+        `first_normed`: the first norm's result, if whoever wrote the residual has formed it already.
         In a step of few rows the parts that offer it fold the norms into their products and add
         their results into the residual themselves; otherwise the norm kernels do both.
         A step that keeps a trace (`ctx.trace`, a dict) leaves there, under `ctx.trace_prefix`, the
@@ -71,6 +110,8 @@ class PreNormBlock:
         residual before) and "output" (the normed inputs are folded away)."""
         trace = getattr(ctx, "trace", None)
         rows = residual.shape[0]
+        if not self.plain:
+            return self._forward_general(residual, pending, ctx, binding, first_normed)
         few = ops.few_rows_route(rows, self.dtype) and (trace is None or getattr(ctx, "trace_serving_route", False))
         if trace is not None and not few:
             return self._forward_traced(residual, pending, ctx, binding)
@@ -97,6 +138,37 @@ class PreNormBlock:
             keep("mlp_output", added)
             keep("output", before + added)
         return out
+
+    def _forward_general(self, residual, pending, ctx, binding, first_normed=None):
+        """A layer without a feed-forward, or with parts between its norms and sublayers: norm, that part, sublayer,
+        one after the other; the last result is handed on.  With a trace: "input_norm" and "post_attention_norm" are
+        what the sublayers read, "attention_output" and "mlp_output" their results, "output" the residual afterwards
+        (the block then adds its last result itself and hands on nothing)."""
+        trace = getattr(ctx, "trace", None)
+
+        def keep(name, tensor):
+            if trace is not None:
+                trace[ctx.trace_prefix + name] = tensor.float().clone()
+        normed = first_normed if first_normed is not None else self.mixer_norm.add_forward(residual, pending)
+        if self.mixer_input is not None:
+            normed = self.mixer_input.forward(normed, ctx, binding.block_state[:, 0])
+        keep("input_norm", normed)
+        out = self.mixer.forward(normed, ctx, binding)
+        if trace is not None:
+            keep("attention_output", as_product(out).dense(torch.float32))
+        if self.feed_forward is not None:
+            normed = self.feed_forward_norm.add_forward(residual, out)
+            if self.feed_forward_input is not None:
+                normed = self.feed_forward_input.forward(normed, ctx, binding.block_state[:, 1])
+            keep("post_attention_norm", normed)
+            out = self.feed_forward.forward(normed, ctx)
+            if trace is not None:
+                keep("mlp_output", as_product(out).dense(torch.float32))
+        if trace is None:
+            return out
+        residual += as_product(out).dense(torch.float32)
+        keep("output", residual)
+        return None
 
     def _forward_traced(self, residual, pending, ctx, binding):
         def keep(name, tensor):

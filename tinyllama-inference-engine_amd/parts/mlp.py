@@ -76,3 +76,38 @@ class GatedMLP(FeedForward):
         if isinstance(hidden, ops.Product):
             hidden = ops.silu_mul(hidden, self.dtype, interleaved=True, gate=self.activation, alpha=self.alpha, limit=self.limit)
         return self.down(hidden, into=into)
+
+
+@register("feed_forward", "mlp")
+class PlainMLP(FeedForward):
+    """down(act(up(x))), no gate.  spec: hidden_size, intermediate_size, activation: "xielu", which has two learned numbers
+    (p, q): for z > 0 softplus(p) z^2 + z / 2, otherwise (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2; names (the tensors'
+    names after the prefix, by role: up, down, act).
+    Tensors: `<prefix>{up,down}_proj.weight`, `<prefix>act` [2] unless `names` says otherwise."""
+    graph_safe = True
+    NAMES = {"up": "up_proj.weight", "down": "down_proj.weight", "act": "act"}
+
+    def __init__(self, spec: PartSpec, dtype, device):
+        super().__init__(spec, dtype, device)
+        self.hidden, self.inter = int(spec["hidden_size"]), int(spec["intermediate_size"])
+        self.activation = spec.get("activation", "xielu")
+        if self.activation != "xielu":
+            raise invalid_config(f"mlp: activation '{self.activation}' is not implemented")
+        self.names = {**self.NAMES, **dict(spec.get("names") or {})}
+        self.up = self.down = self.numbers = None
+
+    @classmethod
+    def tensor_specs(cls, spec, prefix):
+        names = {**cls.NAMES, **dict(spec.get("names") or {})}
+        hidden, inter = int(spec["hidden_size"]), int(spec["intermediate_size"])
+        return [TensorSpec(prefix + names["up"], (inter, hidden)), TensorSpec(prefix + names["down"], (hidden, inter)),
+                TensorSpec(prefix + names["act"], (2,), init="offset")]
+
+    def load(self, weights, prefix):
+        keep = partial(keep_in, weights)
+        self.up = Linear(weights[prefix + self.names["up"]], None, self.dtype, keep=keep)
+        self.down = Linear(weights[prefix + self.names["down"]], None, self.dtype, keep=keep)
+        self.numbers = keep(weights[prefix + self.names["act"]].contiguous())
+
+    def forward(self, x, ctx, into=None):
+        return self.down(ops.xielu(ops.as_product(self.up(x)), self.numbers, self.dtype))

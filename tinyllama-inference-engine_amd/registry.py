@@ -20,9 +20,10 @@ BLOCKS: dict[str, Any] = {}
 EMBEDDINGS: dict[str, Any] = {}
 HEADS: dict[str, Any] = {}
 LAYER_INPUTS: dict[str, Any] = {}
+SUBLAYER_INPUTS: dict[str, Any] = {}
 
 _TABLES = {"architecture": ARCHITECTURES, "mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS,
-           "position_encoding": POSITION_ENCODINGS, "block": BLOCKS, "embedding": EMBEDDINGS, "head": HEADS, "layer_input": LAYER_INPUTS}
+           "position_encoding": POSITION_ENCODINGS, "block": BLOCKS, "embedding": EMBEDDINGS, "head": HEADS, "layer_input": LAYER_INPUTS, "sublayer_input": SUBLAYER_INPUTS}
 
 
 def register(table: str, name: str) -> Callable:

@@ -34,6 +34,7 @@ def random_tensors(specs: list[TensorSpec], seed: int, std: float = 0.02, norm_s
 
 def _draw(spec: TensorSpec, seed: int, std: float, norm_std: float, dtype: torch.dtype, device) -> torch.Tensor:
     generator = _generator(seed, spec.name, device)
+    spec = TensorSpec(spec.name, tuple(spec.free_extent if extent == -1 else extent for extent in spec.shape), spec.init)
     values = torch.randn(spec.shape, generator=generator, dtype=torch.float32, device=device)
     if spec.init == "normal":
         values = values * std
@@ -46,6 +47,12 @@ def _draw(spec: TensorSpec, seed: int, std: float, norm_std: float, dtype: torch
     elif spec.init == "forget_bias":
         # the bias of a forget gate, as such gates are commonly started: between 3 and 6, so that little is forgotten
         values = 3.0 + 3.0 * torch.rand(spec.shape, generator=_generator(seed, spec.name + "#", device), dtype=torch.float32, device=device)
+    elif spec.init == "fraction":
+        values = torch.rand(spec.shape, generator=generator, dtype=torch.float32, device=device)
+    elif spec.init == "mix":
+        # the weights of a sum of which the last summand is the main one
+        values = values * 0.2
+        values[..., -1] += 1.0
     else:
         raise ValueError(f"unknown init '{spec.init}' for {spec.name}")
     return values.to(dtype)
@@ -64,7 +71,7 @@ def resident_random_tensors(specs: list[TensorSpec], seed: int, std: float = 0.0
     for spec in wanted:
         count = 1
         for extent in spec.shape:
-            count *= int(extent)
+            count *= int(spec.free_extent if extent == -1 else extent)
         sizes[spec.name] = count * dtype.itemsize
     return ResidentWeights({spec.name: draw(spec) for spec in wanted}, sizes, device)
 

@@ -23,6 +23,12 @@ from ..errors import EngineError, ErrorCode
 from .safetensors_io import SafetensorsFile
 
 
+def _fits(stored, expected) -> bool:
+    """An expected extent of -1 stands for a size that the file itself gives (any positive one)."""
+    stored, expected = tuple(stored), tuple(expected)
+    return len(stored) == len(expected) and all(want == have or (want == -1 and have > 0) for have, want in zip(stored, expected))
+
+
 class WeightStore:
     """All safetensors files of a model folder behind one `get(name)`."""
 
@@ -106,7 +112,7 @@ class WeightStore:
                       if name not in expected and not any(pattern.fullmatch(name) for pattern in patterns)]
         wrong = []
         for spec in specs:
-            if spec.name in self._where and tuple(self.shape(spec.name)) != tuple(spec.shape):
+            if spec.name in self._where and not _fits(self.shape(spec.name), spec.shape):
                 wrong.append(f"{spec.name}: stored {list(self.shape(spec.name))}, expected {list(spec.shape)}")
         if missing or unexpected or wrong:
             parts = []
