@@ -230,20 +230,57 @@ def raketar_configs(sizes):
     return raketar, llama
 
 
+# layer sizes for `--design tugalix`: the same widths and vocabulary; retention and gated linear attention with heads whose
+# query/key size is half their value size, after the ratios of published retention and gated-linear-attention models (keys
+# half the width, values the width); attention beside token-shift mixing with Llama's heads on the left and heads of 64
+# dims on the right, after published RWKV models; a decay rank of 64; four taps of the convolution; a feed-forward of two
+# matrices at 1.5 times the gated one's inner size (equal weights) in two layers of four
+TUGALIX_SIZES = {
+    "w2048": dict(width=2048, ff=8448, llama_ff=5632, heads=32, kv_heads=4, dim=64, ret_heads=8, ret_dim=128, ret_vdim=256,
+                  gla_heads=4, gla_dim=256, gla_vdim=512, shift_heads=32, shift_dim=64, rank=64, taps=4, vocab=32000),
+    "w4096": dict(width=4096, ff=21504, llama_ff=14336, heads=32, kv_heads=8, dim=128, ret_heads=16, ret_dim=128, ret_vdim=256,
+                  gla_heads=8, gla_dim=256, gla_vdim=512, shift_heads=64, shift_dim=64, rank=64, taps=4, vocab=32000),
+}
+
+
+def tugalix_configs(sizes):
+    """(the Tugalix configuration, the Llama configuration of equal sizes): retention without a feed-forward, attention
+    beside token-shift mixing with one, gated linear attention without, attention beside token-shift mixing with one.
+    Beside four Llama layers of the same width and heads (a Llama layer always has its feed-forward)."""
+    s = sizes
+    dense = {"kind": "dense", "ff": s["ff"]}
+    retention = {"heads": s["ret_heads"], "dim": s["ret_dim"], "vdim": s["ret_vdim"],
+                 "decay": [1.0 - 2.0 ** (-5 - 3 * head / max(s["ret_heads"] - 1, 1)) for head in range(s["ret_heads"])],
+                 "rot": {"base": 10000.0, "dims": s["ret_dim"]}}
+    gla = {"heads": s["gla_heads"], "dim": s["gla_dim"], "vdim": s["gla_vdim"], "tau": 16.0, "rank": s["rank"]}
+    side = {"left": {"heads": s["heads"], "kv_heads": s["kv_heads"], "dim": s["dim"], "vdim": s["dim"], "scale": s["dim"] ** -0.5,
+                     "rot": {"base": 10000.0, "dims": s["dim"]}},
+            "right": {"heads": s["shift_heads"], "dim": s["shift_dim"], "rank": s["rank"]}, "left_scale": 1.0, "right_scale": 1.0}
+    layers = [{"type": "retention", "mixer": retention, "mlp": None}, {"type": "parallel", "mixer": side, "mlp": dense},
+              {"type": "gla", "mixer": gla, "mlp": None}, {"type": "parallel", "mixer": side, "mlp": dense}]
+    tugalix = {"architecture": "Tugalix", "vocab": s["vocab"], "width": s["width"], "norm": {"eps": 1e-5}, "canon": {"taps": s["taps"]},
+               "logit_scale": 1.0, "layers": layers}
+    llama = dict(TINYLLAMA, hidden_size=s["width"], intermediate_size=s["llama_ff"], num_hidden_layers=4,
+                 num_attention_heads=s["heads"], num_key_value_heads=s["kv_heads"], vocab_size=s["vocab"], max_position_embeddings=4096)
+    return tugalix, llama
+
+
 def bench_design(args, torch) -> int:
-    """`--design fadutar|raketar`: one JSON line.  Per size: tokens a second of a prompt step of 2048 tokens and of decode steps
+    """`--design fadutar|raketar|tugalix`: one JSON line.  Per size: tokens a second of a prompt step of 2048 tokens and of decode steps
     at the record's batch and context, for that decoder and for the Llama decoder of equal sizes (random
     weights, bfloat16, through the engine's own loop), and every kernel the design adds alone, beside the like kernel."""
     from tlie_amd import Engine, ops
-    from tlie_amd.kernel_bench import bench_design_kernels, bench_raketar_kernels
+    from tlie_amd.kernel_bench import bench_design_kernels, bench_raketar_kernels, bench_tugalix_kernels
     peaks = ops.measured_peaks("cuda:0")
     record = {"metric": f"{args.design}: prefill and decode tok/s beside the Llama decoder of equal sizes", "unit": "tokens/s",
               "n_gpus": 1, "dtype": "bf16", "data": "synthetic: uniform random token ids, random weights",
               "batch": args.batch, "context": args.context, "measured_peaks": peaks, "sizes": {}}
     steps, warmup = min(args.steps, 48), 4
-    all_sizes, configs = (DESIGN_SIZES, design_configs) if args.design == "fadutar" else (RAKETAR_SIZES, raketar_configs)
+    all_sizes, configs, kernels = {"fadutar": (DESIGN_SIZES, design_configs, bench_design_kernels),
+                                   "raketar": (RAKETAR_SIZES, raketar_configs, bench_raketar_kernels),
+                                   "tugalix": (TUGALIX_SIZES, tugalix_configs, bench_tugalix_kernels)}[args.design]
     for name, sizes in all_sizes.items():
-        entry = {"layers": 4 * sizes["groups"] if args.design == "fadutar" else 6, "sizes": sizes}
+        entry = {"layers": {"fadutar": 4 * sizes.get("groups", 0), "raketar": 6, "tugalix": 4}[args.design], "sizes": sizes}
         for model, config in zip((args.design, "llama"), configs(sizes)):
             engine = Engine(None, dtype="bfloat16", config=config, random_seed=0, max_tokens=args.batch * args.context + 4096,
                             page_size=16, max_requests=args.batch + 1)
@@ -255,7 +292,6 @@ def bench_design(args, torch) -> int:
             entry[f"{model}_decode_ms_step"] = seconds / steps * 1e3
             del engine
             torch.cuda.empty_cache()
-        kernels = bench_design_kernels if args.design == "fadutar" else bench_raketar_kernels
         if not args.no_points:
             entry["kernels"] = kernels(sizes, batch=args.batch, context=args.context, prompt=2048,
                                        hbm_gbs=peaks["stream_read_gbs"], mfma_tflops=peaks["mfma_bf16_tflops"])
@@ -290,7 +326,7 @@ def main() -> int:
                         help="time the kernels of a decode step (--batch, --context) and of a prompt step one by one at the "
                              "shape's layer sizes, each inside a replayed recording that walks through copies of its weights; "
                              "NAME keeps the kernels whose name holds it; prints one JSON line per kernel")
-    parser.add_argument("--design", default=None, choices=["fadutar", "raketar"],
+    parser.add_argument("--design", default=None, choices=["fadutar", "raketar", "tugalix"],
                         help="prefill and decode throughput of that decoder design at layer sizes of real models, beside the Llama "
                              "decoder at equal sizes, and its own kernels alone beside the like kernels (one JSON line of its own)")
     parser.add_argument("--shape", default="tinyllama", choices=["tinyllama", *OTHER_SHAPES],

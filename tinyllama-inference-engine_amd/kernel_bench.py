@@ -484,3 +484,133 @@ def bench_raketar_kernels(sizes: dict, batch: int = 8, context: int = 2048, prom
         times = _timed(lambda i: ops.side_gate(pre, ids, side_table, side, bf), 8, samples)
         row(f"{label}: token input's gate", times, tokens * side * 6)
     return rows
+
+
+def bench_tugalix_kernels(sizes: dict, batch: int = 8, context: int = 2048, prompt: int = 2048, samples: int = 10, device="cuda:0",
+                          hbm_gbs: float = 8000.0, mfma_tflops: float = 2500.0) -> list[dict]:
+    """The kernels that the Tugalix decoder adds, each alone at a layer's sizes, for a decode step of `batch` requests at
+    `context` positions and a prompt step of `prompt` tokens, each beside the like kernel of the closest model (the
+    matrix memory's walk and its heads' norm of the memory layers at the same head sizes, the recurrent layers'
+    convolution, Llama's add + norm, rotation and gate); every row carries the fraction of the roofline its bytes or
+    flops reach (`frac`: of `hbm_gbs` for rows with bytes, of `mfma_tflops` for rows with flops).
+    sizes: width, ff, llama_ff, heads, kv_heads, dim (the attention beside the token-shift mixing); ret_heads, ret_dim,
+    ret_vdim; gla_heads, gla_dim, gla_vdim; shift_heads, shift_dim; rank; taps."""
+    device = torch.device(device)
+    torch.cuda.set_device(device)
+    bf, f32 = torch.bfloat16, torch.float32
+    width, ff, lff, taps, rank = sizes["width"], sizes["ff"], sizes["llama_ff"], sizes["taps"], sizes["rank"]
+    lq, lkv, d = sizes["heads"], sizes["kv_heads"], sizes["dim"]
+    rows = []
+
+    def rand(*shape, scale=0.02, dtype=bf):
+        return (torch.randn(shape, device=device, dtype=f32) * scale).to(dtype)
+
+    def row(name, times, read_bytes=0, flops=0):
+        entry = _row(name, times, read_bytes, flops)
+        if read_bytes:
+            entry["frac"] = round(entry["gbs"] / hbm_gbs, 3)
+        elif flops:
+            entry["frac"] = round(entry["tflops"] / mfma_tflops, 4)
+        rows.append(entry)
+
+    def ints(values):
+        return torch.tensor(values, dtype=torch.int32, device=device)
+
+    for label, tokens, seqs in ((f"decode b{batch}", batch, batch), (f"prompt {prompt}", prompt, 1)):
+        if tokens <= 0:
+            continue
+        decode = seqs == tokens
+        if decode:
+            positions = torch.full((tokens,), context - 1, dtype=torch.int32, device=device)
+            token_seq, seq_start = ints(list(range(tokens))), ints(list(range(tokens + 1)))
+        else:
+            positions = torch.arange(tokens, dtype=torch.int32, device=device)
+            token_seq, seq_start = torch.zeros(tokens, dtype=torch.int32, device=device), ints([0, tokens])
+        seq_slot = ints(list(range(seqs)))
+        token_slot = seq_slot[token_seq.long()].contiguous()
+        ctx = SimpleNamespace(max_new=1 if decode else tokens, token_seq=token_seq, token_slot=token_slot, seq_start=seq_start, seq_slot=seq_slot)
+        # ---- the scans: state [dim x vdim] a head; a token costs 4 flops an element of S ---------------------------
+        scans = (("retention", sizes["ret_heads"], sizes["ret_dim"], sizes["ret_vdim"], "head"),
+                 ("gated linear attention", sizes["gla_heads"], sizes["gla_dim"], sizes["gla_vdim"], "channel"),
+                 ("token-shift mixing", sizes["shift_heads"], sizes["shift_dim"], sizes["shift_dim"], "bonus"))
+        for name, heads, dim, vdim, kind in scans:
+            fused = ops.Product(rand(tokens, 2 * heads * dim + 2 * heads * vdim, scale=1.0, dtype=f32 if kind == "head" else bf), 1)
+            state = torch.zeros((seqs, *ops.decay_scan_state_shape(heads, dim, vdim)), dtype=f32, device=device)
+            options = {}
+            if kind == "head":
+                options["head_decay"] = torch.full((heads,), 0.97, dtype=f32, device=device)
+            else:
+                options["decay"] = torch.rand(tokens, heads * dim, device=device) * 0.1 + 0.9
+            if kind == "bonus":
+                options["bonus"] = rand(heads * dim, scale=1.0, dtype=f32)
+            times = _timed(lambda i: ops.decay_scan((fused, 0), (fused, heads * dim), (fused, 2 * heads * dim), state, seq_start, seq_slot,
+                                                    heads, dim, vdim, max_new=ctx.max_new, **options), 8, samples)
+            state_bytes = seqs * heads * dim * vdim * 4 * 2
+            row(f"{label}: scan of {name}, {heads} heads of {dim} x {vdim}", times, state_bytes if decode else 0,
+                0 if decode else 4.0 * tokens * heads * dim * vdim)
+            # the like kernel: the memory layers' walk at the same head sizes (it also carries a normaliser and a maximum)
+            memory_in = ops.Product(rand(tokens, 2 * heads * dim + 2 * heads * vdim, scale=1.0), 1)
+            gates = rand(tokens, 2 * heads, scale=1.0, dtype=f32) + 3.0
+            memory = torch.zeros((seqs, *ops.mlstm_state_shape(heads, dim, vdim)), dtype=f32, device=device)
+            times = _timed(lambda i: ops.mlstm_scan(memory_in, 0, heads * dim, 2 * heads * dim, gates, memory, seq_start, seq_slot, heads, dim,
+                                                    vdim, 15.0, dim ** -0.5, max_new=ctx.max_new), 8, samples)
+            row(f"{label}: matrix memory's walk at these sizes (the memory layers')", times, state_bytes if decode else 0,
+                0 if decode else 4.0 * tokens * heads * dim * vdim)
+            scanned = rand(tokens, heads * vdim, scale=1.0, dtype=f32)
+            weight = rand(heads * vdim, scale=1.0)
+            times = _timed(lambda i: ops.head_combine(scanned, heads, vdim, 1e-5, bf, weight=None if kind == "head" else weight, gate=fused,
+                                                      gate_col=2 * heads * dim + heads * vdim, gate_kind="silu"), 8, samples)
+            row(f"{label}: heads of {name}: norm and gate", times, tokens * heads * vdim * (4 + 2 + 2))
+            if kind == "head":
+                inv_freq = torch.ones(dim // 2, device=device)
+                product = ops.Product(rand(tokens, 2 * heads * dim + 2 * heads * vdim, scale=1.0), 1)
+                times = _timed(lambda i: ops.rotate_heads(product, 0, positions, inv_freq, dim, 2 * heads, heads, dim, 1.0, dim ** -0.5,
+                                                          tail=heads * vdim), 8, samples)
+                row(f"{label}: rotation of q and k on their way into the scan (floats out)", times, tokens * (2 * heads * dim + heads * vdim) * (2 + 4))
+            else:
+                low = rand(tokens, rank, scale=1.0, dtype=f32)
+                up, bias = rand(heads * dim, rank, scale=0.3), rand(heads * dim, scale=1.0)
+                times = _timed(lambda i: ops.low_rank_decay(low, up, bias, "sigmoid_root" if kind == "channel" else "exp_neg_exp", tau=16.0,
+                                                            inner_tanh=kind == "bonus"), 8, samples)
+                row(f"{label}: decays of {name} from rank {rank}", times, tokens * (rank * 4 + heads * dim * 4) + heads * dim * rank * 2)
+        x = rand(tokens, width, scale=1.0)
+        down = rand(rank, width)
+        times = _timed(lambda i: ops.few_outputs(x, down), 8, samples)
+        row(f"{label}: the decays' inner product, float sums ({rank} outputs)", times, (tokens + rank) * width * 2)
+        # ---- rotation + cache write of the attention beside the token-shift mixing is Llama's own kernel -------------
+        # ---- around a sublayer -------------------------------------------------------------------------------------
+        residual = rand(tokens, width, scale=1.0, dtype=f32)
+        first, second = ops.Product(rand(tokens, width, scale=1.0), 1), ops.Product(rand(tokens, width, scale=1.0), 1)
+        norm_w, norm_b = rand(width, scale=1.0), rand(width, scale=1.0)
+        times = _timed(lambda i: ops.layer_norm(residual, first, norm_w, norm_b, 1e-5, f32), 8, samples)
+        row(f"{label}: add + layer norm, floats out", times, tokens * width * (4 + 4 + 2 + 4))
+        times = _timed(lambda i: ops.layer_norm(residual, ops.ScaledSum(first, 1.0, second, 1.0), norm_w, norm_b, 1e-5, f32), 8, samples)
+        row(f"{label}: add of both sides + layer norm, floats out", times, tokens * width * (4 + 4 + 2 + 2 + 4))
+        history = rand(6, tokens, width, scale=1.0, dtype=f32)
+        mix = rand(4, scale=1.0)
+        times = _timed(lambda i: ops.layer_norm(history[3], first, norm_w, norm_b, 1e-5, f32, history=history, history_count=4,
+                                                history_weight=mix, mixed=history[4]), 8, samples)
+        row(f"{label}: add + sum over four results + layer norm, floats out", times, tokens * width * (4 * 4 + 4 + 2 + 4 + 4))
+        times = _timed(lambda i: ops.add_rmsnorm(residual, first, norm_w, 1e-5, bf), 8, samples)
+        row(f"{label}: add + norm (Llama's)", times, tokens * width * (4 + 4 + 2 + 2))
+        normed = rand(tokens, width, scale=1.0, dtype=f32)
+        tap_w = rand(width, taps, scale=0.3)
+        conv_state = torch.zeros(seqs, max(taps - 1, 1), width, dtype=f32, device=device)
+        times = _timed(lambda i: ops.input_conv(normed, tap_w, conv_state, ctx, bf), 8, samples)
+        row(f"{label}: h + conv(h), {taps} taps", times, tokens * width * (4 + 2) + (seqs * (taps - 1) * width * 8 if decode else 0))
+        conv_in = ops.Product(rand(tokens, width, scale=1.0), 1)
+        lru_state = torch.zeros(seqs, taps, width, dtype=f32, device=device)
+        times = _timed(lambda i: ops.causal_conv(conv_in, 0, tap_w, None, lru_state, token_seq, token_slot, seq_start), 8, samples)
+        row(f"{label}: convolution of {taps} taps (the recurrent layers')", times, tokens * width * (2 + 4) + (seqs * (taps - 1) * width * 8 if decode else 0))
+        mu = torch.rand(5, width, device=device).to(bf)
+        shift_state = torch.zeros(seqs, width, dtype=f32, device=device)
+        times = _timed(lambda i: ops.token_shift(x, mu, shift_state, ctx), 8, samples)
+        row(f"{label}: five blends with the token before", times, tokens * width * (2 + 5 * 2))
+        pre = ops.Product(rand(tokens, ff, scale=1.0), 1)
+        numbers = rand(2, scale=1.0)
+        times = _timed(lambda i: ops.xielu(pre, numbers, bf), 4, samples)
+        row(f"{label}: xIELU", times, tokens * ff * 4)
+        dense_up = ops.Product(rand(tokens, 2 * lff, scale=1.0), 1)
+        times = _timed(lambda i: ops.silu_mul(dense_up, bf, interleaved=True), 4, samples)
+        row(f"{label}: SiLU gate (Llama's)", times, tokens * lff * 6)
+    return rows
