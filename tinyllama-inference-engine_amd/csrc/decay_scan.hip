@@ -237,25 +237,43 @@ decay_carry_kernel(float* __restrict__ parts, float* __restrict__ state, const i
 
 // out[t, c] = decay(z), z = bias[c] + sum_r weight[c, r] * f(low[t, r]); f the identity or tanh.
 // kind 0: sigmoid(z)^(1 / tau), formed as exp(logsigmoid(z) / tau); kind 1: exp(-exp(z)).  Float throughout.
-template <typename W>
+// A workgroup takes TT tokens (their low rows lie in LDS) and a thread a channel for all of them, so that a channel's
+// weights are read once for the tile; a step of few tokens takes tiles of one, for the workgroups' number.
+constexpr int kDecayTokens = 8, kDecayTiledFrom = 64;
+
+template <typename W, int TT>
 __global__ void __launch_bounds__(256)
-low_rank_decay_kernel(const float* __restrict__ low, int inner_tanh, const W* __restrict__ weight, const W* __restrict__ bias,
-                      int kind, float tau, float* __restrict__ out, int channels, int rank) {
-  extern __shared__ float shared_low[];
-  const int t = blockIdx.x;
-  for (int r = threadIdx.x; r < rank; r += blockDim.x) {
-    const float v = low[static_cast<size_t>(t) * rank + r];
-    shared_low[r] = inner_tanh ? tanhf(v) : v;
+low_rank_decay_kernel(const float* __restrict__ low, int nsplit, size_t split_stride, int inner_tanh, const W* __restrict__ weight,
+                      const W* __restrict__ bias, int kind, float tau, float* __restrict__ out, int tokens, int channels, int rank) {
+  extern __shared__ float shared_low[];                // [TT][rank]
+  const int t0 = blockIdx.x * TT;
+  const int count = min(TT, tokens - t0);
+  for (int i = threadIdx.x; i < TT * rank; i += blockDim.x) {
+    const int b = i / rank;
+    const float v = b < count ? sum_splits(low + static_cast<size_t>(t0) * rank + i, nsplit, split_stride) : 0.f;
+    shared_low[i] = inner_tanh ? tanhf(v) : v;
   }
   __syncthreads();
+  const float inv_tau = 1.f / tau;
   for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < channels; c += gridDim.y * blockDim.x) {
-    float z = bias != nullptr ? to_float(bias[c]) : 0.f;
+    float z[TT];
+    const float start = bias != nullptr ? to_float(bias[c]) : 0.f;
+#pragma unroll
+    for (int b = 0; b < TT; ++b) z[b] = start;
     const W* row = weight + static_cast<size_t>(c) * rank;
-    for (int r = 0; r < rank; ++r) z += to_float(row[r]) * shared_low[r];
-    float w;
-    if (kind == 0) w = expf((fminf(z, 0.f) - log1pf(expf(-fabsf(z)))) / tau);
-    else w = expf(-expf(z));
-    out[static_cast<size_t>(t) * channels + c] = w;
+    for (int r = 0; r < rank; ++r) {
+      const float w = to_float(row[r]);
+#pragma unroll
+      for (int b = 0; b < TT; ++b) z[b] += w * shared_low[b * rank + r];
+    }
+#pragma unroll
+    for (int b = 0; b < TT; ++b) {
+      if (b >= count) break;
+      float w;
+      if (kind == 0) w = expf((fminf(z[b], 0.f) - log1pf(expf(-fabsf(z[b])))) * inv_tau);
+      else w = expf(-expf(z[b]));
+      out[static_cast<size_t>(t0 + b) * channels + c] = w;
+    }
   }
 }
 
@@ -271,7 +289,7 @@ rotate_heads_kernel(const D* __restrict__ in, int nsplit, size_t split_stride, i
   const int width = heads * dim + tail, half = rot_dim / 2;
   const D* src = in + static_cast<size_t>(t) * row + col;
   const float position = static_cast<float>(positions[t]);
-  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < width; c += gridDim.y * blockDim.x) {
     float value = sum_splits(src + c, nsplit, split_stride);
     if (c < heads * dim) {
       const int head = c / dim, d = c - head * dim;
@@ -357,21 +375,27 @@ extern "C" int tlie_decay_scan(const void* q, int q_nsplit, long long q_stride, 
   return launch_status();
 }
 
-// low: float [tokens, rank]; weight [channels, rank] and bias [channels] (or null) of w_dtype; out: float [tokens, channels].
-extern "C" int tlie_low_rank_decay(const float* low, int inner_tanh, const void* weight, const void* bias, int w_dtype, int kind,
+// low: a float product [nsplit][tokens][rank]; weight [channels, rank] and bias [channels] (or null) of w_dtype; out: float [tokens, channels].
+extern "C" int tlie_low_rank_decay(const float* low, int nsplit, long long split_stride, int inner_tanh, const void* weight, const void* bias, int w_dtype, int kind,
                                    float tau, float* out, int tokens, int channels, int rank, void* stream) {
-  if (tokens <= 0 || channels <= 0 || rank <= 0 || rank > 4096 || kind < 0 || kind > 1 || (kind == 0 && !(tau > 0.f))) return kBadArgument;
+  if (tokens <= 0 || channels <= 0 || rank <= 0 || rank > 1024 || nsplit < 1 || kind < 0 || kind > 1 || (kind == 0 && !(tau > 0.f))) return kBadArgument;
   int across = (channels + 255) / 256;
   if (across > 64) across = 64;
-  const dim3 grid(tokens, across);
+  const int tile = tokens >= kDecayTiledFrom ? kDecayTokens : 1;
+  const dim3 grid((tokens + tile - 1) / tile, across);
+  const size_t lds = static_cast<size_t>(tile) * rank * sizeof(float);
   hipStream_t s = (hipStream_t)stream;
-  if (w_dtype == kF32)
-    hipLaunchKernelGGL((low_rank_decay_kernel<float>), grid, dim3(256), rank * sizeof(float), s, low, inner_tanh,
-                       (const float*)weight, (const float*)bias, kind, tau, out, channels, rank);
-  else if (w_dtype == kBF16)
-    hipLaunchKernelGGL((low_rank_decay_kernel<bf16>), grid, dim3(256), rank * sizeof(float), s, low, inner_tanh,
-                       (const bf16*)weight, (const bf16*)bias, kind, tau, out, channels, rank);
-  else return kBadArgument;
+#define TLIE_LAUNCH(W, TT)                                                                                             \
+  hipLaunchKernelGGL((low_rank_decay_kernel<W, TT>), grid, dim3(256), lds, s, low, nsplit, (size_t)split_stride, inner_tanh, (const W*)weight, \
+                     (const W*)bias, kind, tau, out, tokens, channels, rank)
+  if (w_dtype == kF32) {
+    if (tile == 1) TLIE_LAUNCH(float, 1);
+    else TLIE_LAUNCH(float, kDecayTokens);
+  } else if (w_dtype == kBF16) {
+    if (tile == 1) TLIE_LAUNCH(bf16, 1);
+    else TLIE_LAUNCH(bf16, kDecayTokens);
+  } else return kBadArgument;
+#undef TLIE_LAUNCH
   return launch_status();
 }
 
@@ -382,11 +406,14 @@ extern "C" int tlie_rotate_heads(const void* in, int dtype, int nsplit, long lon
   if (tokens <= 0 || heads <= 0 || dim <= 0 || rot_dim < 0 || rot_dim > dim || rot_dim % 2 != 0 || tail < 0 || nsplit < 1) return kBadArgument;
   if (col < 0 || col + heads * dim + tail > row || (rot_dim > 0 && inv_freq == nullptr)) return kBadArgument;
   hipStream_t s = (hipStream_t)stream;
+  int across = (heads * dim + tail + 1023) / 1024;       // (about four columns a thread)
+  if (across > 64) across = 64;
+  const dim3 grid(tokens, across);
   if (dtype == kF32)
-    hipLaunchKernelGGL((rotate_heads_kernel<float>), dim3(tokens), dim3(256), 0, s, (const float*)in, nsplit, (size_t)split_stride,
+    hipLaunchKernelGGL((rotate_heads_kernel<float>), grid, dim3(256), 0, s, (const float*)in, nsplit, (size_t)split_stride,
                        row, col, positions, inv_freq, rot_dim, heads, heads_a, dim, scale_a, scale_b, tail, out);
   else if (dtype == kBF16)
-    hipLaunchKernelGGL((rotate_heads_kernel<bf16>), dim3(tokens), dim3(256), 0, s, (const bf16*)in, nsplit, (size_t)split_stride,
+    hipLaunchKernelGGL((rotate_heads_kernel<bf16>), grid, dim3(256), 0, s, (const bf16*)in, nsplit, (size_t)split_stride,
                        row, col, positions, inv_freq, rot_dim, heads, heads_a, dim, scale_a, scale_b, tail, out);
   else return kBadArgument;
   return launch_status();

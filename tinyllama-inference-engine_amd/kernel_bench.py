@@ -574,9 +574,13 @@ def bench_tugalix_kernels(sizes: dict, batch: int = 8, context: int = 2048, prom
                                                             inner_tanh=kind == "bonus"), 8, samples)
                 row(f"{label}: decays of {name} from rank {rank}", times, tokens * (rank * 4 + heads * dim * 4) + heads * dim * rank * 2)
         x = rand(tokens, width, scale=1.0)
-        down = rand(rank, width)
-        times = _timed(lambda i: ops.few_outputs(x, down), 8, samples)
+        from .parts.linear import Linear
+        down = Linear(rand(rank, width), None, bf)
+        times = _timed(lambda i: down(x, out_dtype=f32), 8, samples)
         row(f"{label}: the decays' inner product, float sums ({rank} outputs)", times, (tokens + rank) * width * 2)
+        gate_w = rand(rank, width)
+        times = _timed(lambda i: ops.few_outputs(x, gate_w), 8, samples)
+        row(f"{label}: a product of {rank} outputs with float sums (the memory layers' gates')", times, (tokens + rank) * width * 2)
         # ---- rotation + cache write of the attention beside the token-shift mixing is Llama's own kernel -------------
         # ---- around a sublayer -------------------------------------------------------------------------------------
         residual = rand(tokens, width, scale=1.0, dtype=f32)

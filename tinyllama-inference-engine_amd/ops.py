@@ -858,27 +858,28 @@ def rotate_heads(fused: Product, col: int, positions: torch.Tensor, inv_freq: to
 LOW_RANK_DECAYS = {"sigmoid_root": 0, "exp_neg_exp": 1}
 
 
-def low_rank_decay(low: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, kind: str, tau: float = 1.0,
+def low_rank_decay(low, weight: torch.Tensor, bias: torch.Tensor | None, kind: str, tau: float = 1.0,
                    inner_tanh: bool = False) -> torch.Tensor:
     """Decays per token and channel from a low-rank product: z = bias + weight . f(low) (f: tanh or the identity), then
-    "sigmoid_root": sigmoid(z)^(1 / tau); "exp_neg_exp": exp(-exp(z)).  low: float32 [tokens, rank]; weight [channels, rank].
-    Float throughout; returns float32 [tokens, channels]."""
-    _device_tensor(low, "low", torch.float32)
+    "sigmoid_root": sigmoid(z)^(1 / tau); "exp_neg_exp": exp(-exp(z)).  low: a float32 product [tokens, rank] (a tensor,
+    or a `Product` of float partial sums); weight [channels, rank].  Float throughout; returns float32 [tokens, channels]."""
+    low = as_product(low)
+    _check_product(low, "low")
     _device_tensor(weight, "weight", (torch.float32, torch.bfloat16))
-    if low.dim() != 2 or weight.dim() != 2 or weight.shape[1] != low.shape[1] or low.shape[1] > 4096:
-        raise invalid_shape("low_rank_decay: low [tokens, rank], weight [channels, rank], rank up to 4096")
+    if low.data.dtype != torch.float32 or weight.dim() != 2 or weight.shape[1] != low.cols or low.cols > 1024:
+        raise invalid_shape("low_rank_decay: low float32 [tokens, rank], weight [channels, rank], rank up to 1024")
     if bias is not None:
         _device_tensor(bias, "bias", weight.dtype)
         if bias.shape != (weight.shape[0],):
             raise invalid_shape("low_rank_decay: one bias a channel")
     if kind not in LOW_RANK_DECAYS or (kind == "sigmoid_root" and not tau > 0.0):
         raise invalid_argument("low_rank_decay: an unknown kind, or a root that is not positive")
-    out = torch.empty((low.shape[0], weight.shape[0]), dtype=torch.float32, device=low.device)
-    if low.shape[0] == 0:
+    out = torch.empty((low.rows, weight.shape[0]), dtype=torch.float32, device=low.data.device)
+    if low.rows == 0:
         return out
-    _check(library().tlie_low_rank_decay(_ptr(low), int(inner_tanh), _ptr(weight), _ptr(bias), dtype_code(weight.dtype),
-                                         LOW_RANK_DECAYS[kind], ctypes.c_float(tau), _ptr(out), low.shape[0], weight.shape[0],
-                                         low.shape[1], _stream()), "low_rank_decay")
+    _check(library().tlie_low_rank_decay(_ptr(low.data), low.nsplit, ctypes.c_longlong(low.split_stride), int(inner_tanh), _ptr(weight),
+                                         _ptr(bias), dtype_code(weight.dtype), LOW_RANK_DECAYS[kind], ctypes.c_float(tau), _ptr(out),
+                                         low.rows, weight.shape[0], low.cols, _stream()), "low_rank_decay")
     return out
 
 

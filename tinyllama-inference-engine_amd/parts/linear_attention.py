@@ -138,9 +138,9 @@ class GatedLinearAttention(Mixer):
         keep = partial(keep_in, weights)
         get = lambda role: weights[prefix + self.names[role]]        # noqa: E731
         self.fused = Linear(torch.cat([get("q"), get("k"), get("v"), get("gate")], dim=0).contiguous(), None, self.dtype, keep=keep)
-        self.down = keep(get("decay_down").contiguous())
+        self.down = Linear(get("decay_down"), None, self.dtype, keep=keep)
         self.up = keep(get("decay_up").contiguous())
-        if self.down.shape[0] != self.up.shape[1]:
+        if self.down.out_features != self.up.shape[1]:
             raise invalid_config("gated_linear_attention: the decay's two matrices do not share their inner size")
         self.up_bias = keep(get("decay_bias").to(self.up.dtype).contiguous())
         self.norm = keep(get("norm").repeat(self.heads).contiguous())         # (one entry a head and dim, as the combine kernel reads it)
@@ -152,7 +152,8 @@ class GatedLinearAttention(Mixer):
     def forward(self, x, ctx, binding: Binding, into=None):
         fused = ops.as_product(self.fused(x))
         keys, values = self.heads * self.d, self.heads * self.dv
-        decay = ops.low_rank_decay(ops.few_outputs(x, self.down), self.up, self.up_bias, "sigmoid_root", tau=self.tau)
+        # (the inner product's sums stay float: what enters the decay is not rounded on its way)
+        decay = ops.low_rank_decay(self.down(x, out_dtype=torch.float32), self.up, self.up_bias, "sigmoid_root", tau=self.tau)
         scanned = ops.decay_scan((fused, 0), (fused, keys), (fused, 2 * keys), binding.state, ctx.seq_start, ctx.seq_slot,
                                  self.heads, self.d, self.dv, decay=decay, q_scale=float(self.d) ** -0.5, max_new=ctx.max_new)
         normed = ops.head_combine(scanned, self.heads, self.dv, self.eps, self.dtype, weight=self.norm, gate=fused,
@@ -198,9 +199,9 @@ class TokenShiftMixing(Mixer):
         get = lambda role: weights[prefix + self.names[role]]        # noqa: E731
         self.blends = keep(torch.stack([get("shift_" + blend) for blend in self.BLENDS], dim=0).contiguous())
         self.products = [Linear(get(role), None, self.dtype, keep=keep) for role in ("r", "k", "v", "gate")]
-        self.down = keep(get("decay_down").contiguous())
+        self.down = Linear(get("decay_down"), None, self.dtype, keep=keep)
         self.up = keep(get("decay_up").contiguous())
-        if self.down.shape[0] != self.up.shape[1]:
+        if self.down.out_features != self.up.shape[1]:
             raise invalid_config("token_shift_mixing: the decay's two matrices do not share their inner size")
         self.base = keep(get("decay_base").to(self.up.dtype).contiguous())
         self.bonus = keep(get("bonus").float().reshape(-1).contiguous())        # (it enters the scan, which is float)
@@ -218,7 +219,7 @@ class TokenShiftMixing(Mixer):
         before = binding.state[:, scan_floats:]
         blended = ops.token_shift(x, self.blends, before, ctx)
         r, k, v, gate = (ops.as_product(product(blended[index])) for index, product in enumerate(self.products))
-        decay = ops.low_rank_decay(ops.few_outputs(blended[4], self.down), self.up, self.base, "exp_neg_exp", inner_tanh=True)
+        decay = ops.low_rank_decay(self.down(blended[4], out_dtype=torch.float32), self.up, self.base, "exp_neg_exp", inner_tanh=True)
         scanned = ops.decay_scan((r, 0), (k, 0), (v, 0), binding.state, ctx.seq_start, ctx.seq_slot, self.heads, self.d, self.d,
                                  decay=decay, bonus=self.bonus, max_new=ctx.max_new)
         normed = ops.head_combine(scanned, self.heads, self.d, self.eps, self.dtype, weight=self.norm, gate=gate, gate_col=0,
