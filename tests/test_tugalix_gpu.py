@@ -783,12 +783,20 @@ def test_the_command_line_and_the_replay_program_run_the_design(setups, tmp_path
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("which", ["two_attentions", "equal_sizes"])
+@pytest.mark.parametrize("which", ["two_attentions", "equal_sizes", "odd_sizes"])
 def test_models_of_other_orders_and_sizes(tmp_path, which, dtype):
     """Two layers with attention after each other (two page groups' worth of caches) at a width that is no multiple of 8;
-    and a model whose sizes are all equal (heads' dims, values, width over heads, the inner size), which would hide
-    two sizes taken for each other, next to one whose sizes all differ."""
-    if which == "two_attentions":
+    a model whose sizes are all equal (heads' dims, values, width over heads, the inner size), which would hide
+    two sizes taken for each other, next to one whose sizes all differ; and one whose width, vocabulary, heads' sizes
+    and inner sizes are all odd or twice an odd number (no kernel's wide form fits), with eight taps."""
+    if which == "odd_sizes":
+        raw = {"architecture": "Tugalix", "vocab": 61, "width": 54, "norm": {"eps": 1e-5}, "canon": {"taps": 8}, "logit_scale": 0.9,
+               "layers": [{"type": "parallel", "mixer": _side_mixer({"left": (3, 1, 6, 5, 0.4, 300.0, 2), "right": (3, 9, 5), "scales": (0.9, 1.1)}),
+                           "mlp": {"kind": "dense", "ff": 35}},
+                          {"type": "gla", "mixer": {"heads": 3, "dim": 7, "vdim": 9, "tau": 2.5, "rank": 3}, "mlp": None},
+                          {"type": "retention", "mixer": {"heads": 5, "dim": 10, "vdim": 3, "decay": [0.5, 0.9, 0.99, 0.999, 0.8],
+                                                          "rot": {"base": 1000.0, "dims": 6}}, "mlp": {"kind": "dense", "ff": 27}}]}
+    elif which == "two_attentions":
         raw = {"architecture": "Tugalix", "vocab": 77, "width": 100, "norm": {"eps": 1e-5}, "canon": {"taps": 3}, "logit_scale": 1.5,
                "layers": [{"type": "parallel", "mixer": _side_mixer(SIDES[0]), "mlp": {"kind": "dense", "ff": 52}},
                           {"type": "parallel", "mixer": _side_mixer(SIDES[1]), "mlp": None},
