@@ -55,6 +55,13 @@ class LayerSpec:
     sublayer_input: PartSpec | None = None
     mixer_input_place: str = "mixer_input."
     feed_forward_input_place: str = "feed_forward_input."
+    # for the arrangement on a residual of several streams ("hyper_connections"): how many streams (the model's
+    # `ModelSpec.streams`), and the places of each sublayer's three tensors: `in` [S] (what the sublayer reads: a weighted
+    # sum of the streams), `mix` [S, S] ([from, to]: how the streams are mixed among themselves) and `out` [S] (how much of
+    # the sublayer's result each stream takes)
+    streams: int = 0
+    mixer_streams_place: str = "mixer_streams."
+    feed_forward_streams_place: str = "feed_forward_streams."
 
 
 @dataclass(frozen=True)
@@ -103,11 +110,19 @@ class ModelSpec:
     ignored_tensors: tuple[str, ...] = ()
     # tensors that belong to no single part: tables that several layers read a part of each, the vectors that runs add
     shared_tensors: tuple["TensorSpec", ...] = ()
+    # 0: one residual per token.  S > 0: S streams of it, all equal to the embedding's output at the start, which the
+    # layers (of an arrangement made for streams) read from and write to; their sum is what the final norm reads.
+    streams: int = 0
 
     def validate(self) -> None:
         from ..errors import invalid_config
         if not self.runs:
             raise invalid_config("a model needs at least one layer to run")
+        for layer in self.layers:
+            if layer.streams != self.streams:
+                raise invalid_config("every layer works on as many streams of the residual as the model has")
+        if self.streams and any(run.add_embedding or run.add_vector is not None or run.depth_mix is not None for run in self.runs):
+            raise invalid_config("runs that add something to the residual do not go with a residual of several streams")
         for index, run in enumerate(self.runs):
             if not 0 <= run.layer < len(self.layers):
                 raise invalid_config(f"run {index} names layer {run.layer}, which does not exist")
@@ -134,6 +149,6 @@ class TensorSpec:
     that the file gives and no configuration names (random weights draw `free_extent` there)."""
     name: str
     shape: tuple[int, ...]
-    init: str = "normal"        # how random weights draw it: "normal", "norm" (around 1), "offset" (a norm's weight stored around 0), "zeros", "forget_bias" (between 3 and 6), "fraction" (between 0 and 1), "mix" (weights of a sum: the last near 1, the others near 0)
+    init: str = "normal"        # how random weights draw it: "normal", "norm" (around 1), "offset" (a norm's weight stored around 0), "zeros", "forget_bias" (between 3 and 6), "fraction" (between 0 and 1), "mix" (weights of a sum: the last near 1, the others near 0), "near_identity" (a square matrix: 1 on the diagonal, small elsewhere), "share" (numbers around 1 / count)
     free_extent: int = 16
     optional: bool = False       # absent is no error, present it is checked and not read (a tied head's matrix that some files still carry)

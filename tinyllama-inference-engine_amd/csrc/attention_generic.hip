@@ -26,6 +26,7 @@ namespace tlie {
 // counted from position 0 of the sequence).
 // sink (or null): one number per query head that joins the softmax's denominator as exp(sink): it has
 // no key and no value and is not scaled.
+// softcap > 0: a scaled score s becomes softcap * tanh(s / softcap) before the softmax.
 // A workgroup of 256 threads serves one (token, head).  Its threads form 256 / CHUNK groups of
 // CHUNK threads (CHUNK >= d); chunk c of the context (keys c * CHUNK ..) belongs to group
 // c % groups, and every group keeps a running maximum, sum and output of its own over its chunks,
@@ -47,7 +48,7 @@ __global__ void __launch_bounds__(256)
 attention_generic_kernel(const T* __restrict__ q, const T* __restrict__ cache, const int* __restrict__ block_table,
                          int max_blocks, const int* __restrict__ token_seq, const int* __restrict__ positions,
                          T* __restrict__ out, int nq, int nkv, int d, int dv, int page_size, int window, int chunk,
-                         const float* __restrict__ sink, float scale,
+                         const float* __restrict__ sink, float scale, float softcap,
                          const int* __restrict__ seq_start, int min_tokens, int vshare, int out_f32) {
   constexpr int kGroups = 256 / CHUNK, kWavesPerGroup = CHUNK / 64;
   if (seq_start != nullptr) {                      // (the same for the whole workgroup)
@@ -117,6 +118,7 @@ attention_generic_kernel(const T* __restrict__ q, const T* __restrict__ cache, c
       }
       for (; i < d; ++i) dot += q_row[i] * to_float(key[i]);
       score = dot * scale;
+      if (softcap > 0.f) score = softcap * tanhf(score / softcap);
     }
     const float new_max = fmaxf(running_max, over_group(score, true));
     const float p = valid ? expf(score - new_max) : 0.f;
@@ -204,7 +206,7 @@ __global__ void __launch_bounds__(64 * kTiledWaves)
 attention_generic_tiled_kernel(const T* __restrict__ q, const T* __restrict__ cache, const int* __restrict__ block_table,
                                int max_blocks, const int* __restrict__ token_seq, const int* __restrict__ positions,
                                T* __restrict__ out, int tokens, int nq, int nkv, int d, int dv, int page_size, int window,
-                               int chunk, const float* __restrict__ sink, float scale, int tokens_per_block, int heads_per_block, const int* __restrict__ seq_start, int min_tokens,
+                               int chunk, const float* __restrict__ sink, float scale, float softcap, int tokens_per_block, int heads_per_block, const int* __restrict__ seq_start, int min_tokens,
                                int vshare, int out_f32) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   // rows of a multiple of 4 floats, so that four values are one LDS read, plus 4: a wave's lanes, each
@@ -332,7 +334,7 @@ attention_generic_tiled_kernel(const T* __restrict__ q, const T* __restrict__ ca
             const bool column = col_tok[s] >= run_first && col_tok[s] < run_end && col_pos[s] >= start && col_lo[s] < start + 64;   // a chunk without keys changes nothing
             if (!column) continue;                 // (uniform over the wave)
             const bool valid = j >= col_lo[s] && j <= col_pos[s];
-            const float score = valid ? dot[u] * scale : -INFINITY;
+            const float score = valid ? (softcap > 0.f ? softcap * tanhf(dot[u] * scale / softcap) : dot[u] * scale) : -INFINITY;
             const float new_max = fmaxf(run_max[g][s], wave_max(score));
             const float p = valid ? expf(score - new_max) : 0.f;
             my_prob[u * 64 + lane] = p;
@@ -413,14 +415,14 @@ extern "C" int tlie_attention_generic(const void* q, const void* cache, int dtyp
                                       int max_blocks, const int* token_seq, const int* positions, void* out,
                                       int tokens, int nq, int nkv, int d, int dv, int page_size, int window, int chunk,
                                       const float* sink, float scale, int tiled, const int* seq_start, int min_tokens,
-                                      int vshare, int out_f32, void* stream) {
+                                      int vshare, int out_f32, float softcap, void* stream) {
   // tiled 0: the kernel of one (token, head) a workgroup; 1: the kernel that shares keys among a
   // sequence's tokens (head sizes up to 64); 2: both, each token served by one of them: the second
   // takes the sequences that bring min_tokens tokens or more (seq_start: int32 [sequences + 1], the
   // step's cumulative token counts), the first the others.  A token gets the same bits from either.
   // (d only bounds the length of a dot product; dv is served by one thread a dim of a group of at most 256)
   if (tokens <= 0 || nq <= 0 || nkv <= 0 || nq % nkv != 0 || d <= 0 || d > 4096 || dv <= 0 || dv > 256 || page_size <= 0 ||
-      max_blocks <= 0 || chunk < 0 || vshare <= 0 || nkv % vshare != 0)
+      max_blocks <= 0 || chunk < 0 || vshare <= 0 || nkv % vshare != 0 || softcap < 0.f)
     return kBadArgument;
   if (tiled < 0 || tiled > 2 || (tiled == 2 && (seq_start == nullptr || min_tokens < 1))) return kBadArgument;
   if (dtype != kF32 && dtype != kBF16) return kBadArgument;
@@ -437,11 +439,11 @@ extern "C" int tlie_attention_generic(const void* q, const void* cache, int dtyp
     if (dtype == kF32)
       hipLaunchKernelGGL((attention_generic_tiled_kernel<float>), grid, dim3(64 * kTiledWaves), bytes, (hipStream_t)stream, (const float*)q,
                          (const float*)cache, block_table, max_blocks, token_seq, positions, (float*)out, tokens, nq, nkv, d, dv,
-                         page_size, window, chunk, sink, scale, tokens_per_block, heads_per_block, select, min_tokens, vshare, out_f32);
+                         page_size, window, chunk, sink, scale, softcap, tokens_per_block, heads_per_block, select, min_tokens, vshare, out_f32);
     else
       hipLaunchKernelGGL((attention_generic_tiled_kernel<bf16>), grid, dim3(64 * kTiledWaves), bytes, (hipStream_t)stream, (const bf16*)q,
                          (const bf16*)cache, block_table, max_blocks, token_seq, positions, (bf16*)out, tokens, nq, nkv, d, dv,
-                         page_size, window, chunk, sink, scale, tokens_per_block, heads_per_block, select, min_tokens, vshare, out_f32);
+                         page_size, window, chunk, sink, scale, softcap, tokens_per_block, heads_per_block, select, min_tokens, vshare, out_f32);
     const int status = launch_status();
     if (status != kOk || tiled == 1) return status;
   }
@@ -456,7 +458,7 @@ extern "C" int tlie_attention_generic(const void* q, const void* cache, int dtyp
 #define TLIE_LAUNCH(T, CHUNK)                                                                                         \
   hipLaunchKernelGGL((attention_generic_kernel<T, CHUNK>), dim3(tokens, nq), dim3(256), lds, s, (const T*)q,           \
                      (const T*)cache, block_table, max_blocks, token_seq, positions, (T*)out, nq, nkv, d, dv, page_size, \
-                     window, chunk, sink, scale, select, min_tokens, vshare, out_f32)
+                     window, chunk, sink, scale, softcap, select, min_tokens, vshare, out_f32)
   if (dtype == kF32) {
     if (keys == 64) TLIE_LAUNCH(float, 64); else if (keys == 128) TLIE_LAUNCH(float, 128); else TLIE_LAUNCH(float, 256);
   } else if (dtype == kBF16) {

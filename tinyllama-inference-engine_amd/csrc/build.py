@@ -18,7 +18,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 SOURCES = ["elementwise.hip", "rope_cache.hip", "attention_generic.hip", "attention_mfma.hip", "gemm_generic.hip",
            "gemm_skinny.hip", "gemm_rows.hip", "gemm_tiles.hip", "sampling.hip", "library_gemm.hip", "probes.hip",
            "block_linear.hip", "latent.hip", "recurrence.hip", "heads.hip", "mlstm.hip", "routing.hip", "side.hip",
-           "decay_scan.hip", "canon.hip"]
+           "decay_scan.hip", "canon.hip", "streams.hip"]
 HEADERS = ["common.h", "no_alloc.h"]
 LIBRARY = "libtlie_hip.so"
 FLAGS = ["-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-shared",

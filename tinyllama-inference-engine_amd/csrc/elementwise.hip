@@ -256,6 +256,26 @@ __global__ void add_bias_kernel(const float* __restrict__ product, const B* __re
     out[i] = from_float<O>(product[i] + to_float(bias[i % cols]));
 }
 
+// ---- values[t, c] *= sigmoid(pre[t, col + c]): a gate on a mixer's heads, its pre-activations columns col .. col + cols - 1
+// of a wider product (row_width columns a row); the sigmoid and the product float -------------------------------------
+template <typename D, typename A>
+__global__ void sigmoid_gate_kernel(A* __restrict__ values, const D* __restrict__ pre, int nsplit, size_t split_stride,
+                                    int col, int row_width, size_t total, int cols) {
+  for (size_t index = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; index < total;
+       index += static_cast<size_t>(gridDim.x) * blockDim.x) {
+    const size_t t = index / cols, c = index % cols;
+    const float z = sum_splits(pre + t * row_width + col + c, nsplit, split_stride);
+    values[index] = from_float<A>(to_float(values[index]) / (1.f + expf(-z)));
+  }
+}
+
+// ---- x <- cap * tanh(x / cap), in place (capped logits) --------------------------------------------------------------
+__global__ void softcap_kernel(float* __restrict__ x, size_t total, float cap) {
+  for (size_t index = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; index < total;
+       index += static_cast<size_t>(gridDim.x) * blockDim.x)
+    x[index] = cap * tanhf(x[index] / cap);
+}
+
 }  // namespace tlie
 
 using namespace tlie;
@@ -417,4 +437,33 @@ extern "C" int tlie_add_bias(const float* product, const void* bias, int bias_dt
   TLIE_CASE(kBF16, bf16, kBF16, bf16)
 #undef TLIE_CASE
   return kBadArgument;
+}
+
+// values: [rows, cols] of act_dtype, changed in place; pre: a product [nsplit][rows][row_width] whose columns
+// col .. col + cols - 1 are the gate's pre-activations.
+extern "C" int tlie_sigmoid_gate(void* values, int act_dtype, const void* pre, int pre_dtype, int nsplit, long long split_stride,
+                                 int col, int row_width, int rows, int cols, void* stream) {
+  if (rows <= 0 || cols <= 0 || col < 0 || col + cols > row_width || nsplit < 1) return kBadArgument;
+  const size_t total = static_cast<size_t>(rows) * cols;
+  const int blocks = static_cast<int>((total + 255) / 256 < 16384 ? (total + 255) / 256 : 16384);
+  hipStream_t s = (hipStream_t)stream;
+#define TLIE_CASE(DC, D, AC, A)                                                                                  \
+  if (pre_dtype == DC && act_dtype == AC) {                                                                      \
+    hipLaunchKernelGGL((sigmoid_gate_kernel<D, A>), dim3(blocks), dim3(256), 0, s, (A*)values, (const D*)pre, nsplit, \
+                       (size_t)split_stride, col, row_width, total, cols);                                       \
+    return launch_status();                                                                                      \
+  }
+  TLIE_CASE(kF32, float, kF32, float)
+  TLIE_CASE(kF32, float, kBF16, bf16)
+  TLIE_CASE(kBF16, bf16, kBF16, bf16)
+#undef TLIE_CASE
+  return kBadArgument;
+}
+
+extern "C" int tlie_softcap(float* x, long long total, float cap, void* stream) {
+  if (total <= 0 || !(cap > 0.f)) return kBadArgument;
+  const long long wanted = (total + 255) / 256;
+  hipLaunchKernelGGL(softcap_kernel, dim3(static_cast<unsigned>(wanted < 16384 ? wanted : 16384)), dim3(256), 0, (hipStream_t)stream,
+                     x, static_cast<size_t>(total), cap);
+  return launch_status();
 }

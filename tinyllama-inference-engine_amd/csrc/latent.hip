@@ -28,15 +28,15 @@ __global__ void latent_place_kernel(const D* __restrict__ fused, int nsplit, siz
                                     const int* __restrict__ positions, const int* __restrict__ slot_map,
                                     const float* __restrict__ inv_freq, const W* __restrict__ norm_weight, float eps,
                                     A* __restrict__ q_plain, A* __restrict__ q_wide, A* __restrict__ cache, int heads,
-                                    int plain, int rot, int turn, int rank, int value_rows, int page_size) {
+                                    int plain, int rot, int turn, int rank, int value_rows, int page_size, int row_width) {
   extern __shared__ float lds[];
   const int half = turn / 2;
   float* cosines = lds;                  // half
   float* sines = cosines + half;         // half
   float* scratch = sines + half;         // 16
   const int t = blockIdx.x;
-  const int per_head = plain + rot, q_width = heads * per_head, width = q_width + rank + rot, key = rank + rot;
-  const D* in = fused + static_cast<size_t>(t) * width;
+  const int per_head = plain + rot, q_width = heads * per_head, key = rank + rot;
+  const D* in = fused + static_cast<size_t>(t) * row_width;        // (a row may hold more columns after these: someone else's)
   const float pos = static_cast<float>(positions[t]);
   for (int i = threadIdx.x; i < half; i += blockDim.x) sincosf(pos * inv_freq[i], &sines[i], &cosines[i]);
   float square = 0.f;
@@ -82,12 +82,13 @@ using namespace tlie;
 extern "C" int tlie_latent_place(const void* fused, int in_dtype, int nsplit, long long split_stride, const int* positions,
                                  const int* slot_map, const float* inv_freq, const void* norm_weight, int weight_dtype,
                                  float eps, void* q_plain, void* q_wide, void* cache, int act_dtype, int tokens, int heads,
-                                 int plain, int rot, int turn, int rank, int value_rows, int page_size, void* stream) {
+                                 int plain, int rot, int turn, int rank, int value_rows, int page_size, int row_width, void* stream) {
   if (tokens <= 0 || heads <= 0 || plain <= 0 || rot < 0 || turn < 0 || turn > rot || turn % 2 != 0 || rank <= 0 || page_size <= 0 ||
       nsplit < 1)
     return kBadArgument;
   if (value_rows != rank && value_rows != rank + rot) return kBadArgument;
   if (turn > 0 && inv_freq == nullptr) return kBadArgument;
+  if (row_width < heads * (plain + rot) + rank + rot) return kBadArgument;
   const int widest = heads * (plain + rot);
   const int threads = widest >= 1024 ? 1024 : (widest >= 256 ? 256 : 64);
   const size_t lds = (static_cast<size_t>(rot) + 16) * sizeof(float);
@@ -96,7 +97,7 @@ extern "C" int tlie_latent_place(const void* fused, int in_dtype, int nsplit, lo
   if (in_dtype == DC && weight_dtype == WC && act_dtype == AC) {                                                     \
     hipLaunchKernelGGL((latent_place_kernel<D, W, A>), dim3(tokens), dim3(threads), lds, s, (const D*)fused, nsplit,   \
                        (size_t)split_stride, positions, slot_map, inv_freq, (const W*)norm_weight, eps, (A*)q_plain,  \
-                       (A*)q_wide, (A*)cache, heads, plain, rot, turn, rank, value_rows, page_size);                                   \
+                       (A*)q_wide, (A*)cache, heads, plain, rot, turn, rank, value_rows, page_size, row_width);                                   \
     return launch_status();                                                                                          \
   }
   TLIE_CASE(kF32, float, kF32, float, kF32, float)

@@ -143,41 +143,91 @@ __global__ void rope_cache_wide_kernel(const D* __restrict__ qkv, const int* __r
 // [row][d] and after them nkv planes of values [dv][row]), or no key and value heads at all (nkv = 0: the
 // layer reads another layer's cache and only its queries are placed).  Columns in natural order; a
 // rotated element reads its partner's summands itself.  One block a token.
+// Options (each off when its pointer is null or its number zero):
+//   q_norm, k_norm   float weights [nq * d], [nkv * d]: all of a token's query columns together (and all of its key
+//                    columns together) are divided by their root mean square, eps inside the root, and multiplied by
+//                    the weight, before the rotation
+//   values_are_keys  the product has no value columns: a key head's columns as projected (before norm and rotation)
+//                    are also its value head (nv = nkv, dv = d)
+//   temp_coef, temp_every   a query at position p is multiplied by 1 + temp_coef * ln(floor((p + 1) / temp_every) + 1)
+struct PlaceOptions {
+  const float* q_norm;
+  const float* k_norm;
+  float eps;
+  int values_are_keys;
+  float temp_coef;
+  float temp_every;
+};
+
 template <typename D, typename A>
 __global__ void qkv_place_kernel(const D* __restrict__ qkv, int nsplit, size_t split_stride,
                                  const int* __restrict__ positions, const int* __restrict__ slot_map,
                                  const float* __restrict__ inv_freq, int rot_dim, A* __restrict__ q_out,
-                                 A* __restrict__ cache, int nq, int nkv, int nv, int d, int dv, int page_size, int row_width) {
+                                 A* __restrict__ cache, int nq, int nkv, int nv, int d, int dv, int page_size, int row_width,
+                                 PlaceOptions options) {
   extern __shared__ float lds[];
   const int half = rot_dim / 2;
   float* cosines = lds;                  // half
   float* sines = cosines + half;         // half
+  float* scratch = sines + half;         // 16
   const int t = blockIdx.x;
-  const int rotated = (nq + nkv) * d, width = rotated + nv * dv;
+  const int rotated = (nq + nkv) * d, width = rotated + (options.values_are_keys ? 0 : nv * dv);
+  const D* in = qkv + static_cast<size_t>(t) * row_width;
   if (inv_freq != nullptr) {
     const float pos = static_cast<float>(positions[t]);
     for (int i = threadIdx.x; i < half; i += blockDim.x) sincosf(pos * inv_freq[i], &sines[i], &cosines[i]);
     __syncthreads();
   }
+  float q_scale = 1.f, k_scale = 1.f;
+  if (options.q_norm != nullptr) {
+    float square = 0.f;
+    for (int c = threadIdx.x; c < nq * d; c += blockDim.x) {
+      const float v = sum_splits(in + c, nsplit, split_stride);
+      square += v * v;
+    }
+    q_scale = rsqrtf(block_sum(square, scratch) / static_cast<float>(nq * d) + options.eps);
+  }
+  if (options.k_norm != nullptr && nkv > 0) {
+    float square = 0.f;
+    for (int c = nq * d + threadIdx.x; c < rotated; c += blockDim.x) {
+      const float v = sum_splits(in + c, nsplit, split_stride);
+      square += v * v;
+    }
+    k_scale = rsqrtf(block_sum(square, scratch) / static_cast<float>(nkv * d) + options.eps);
+  }
+  if (options.temp_every > 0.f)
+    q_scale *= 1.f + options.temp_coef * logf(floorf(static_cast<float>(positions[t] + 1) / options.temp_every) + 1.f);
+  // a column of q or k after its norm (and, for a query, its temperature), before the rotation
+  auto normed = [&](int c) {
+    const float v = sum_splits(in + c, nsplit, split_stride);
+    if (c < nq * d) return options.q_norm != nullptr ? v * q_scale * options.q_norm[c] : v * q_scale;
+    return options.k_norm != nullptr ? v * k_scale * options.k_norm[c - nq * d] : v;
+  };
   const int slot = nkv > 0 ? slot_map[t] : -1;
   A* page = cache + static_cast<size_t>(slot < 0 ? 0 : slot / page_size) * page_size * (static_cast<size_t>(nkv) * d + static_cast<size_t>(nv) * dv);
   const int row = slot < 0 ? 0 : slot % page_size;
-  const D* in = qkv + static_cast<size_t>(t) * row_width;
   for (int c = threadIdx.x; c < width; c += blockDim.x) {
     if (c >= nq * d && slot < 0) break;  // (columns only grow: what is left is keys and values too)
-    float v = sum_splits(in + c, nsplit, split_stride);
     if (c >= rotated) {
       const int head = (c - rotated) / dv, e = (c - rotated) % dv;
-      page[static_cast<size_t>(nkv) * page_size * d + (static_cast<size_t>(head) * dv + e) * page_size + row] = from_float<A>(v);
+      page[static_cast<size_t>(nkv) * page_size * d + (static_cast<size_t>(head) * dv + e) * page_size + row] =
+          from_float<A>(sum_splits(in + c, nsplit, split_stride));
       continue;
     }
     const int head = c / d, e = c % d;
+    float v = normed(c);
     if (inv_freq != nullptr && e < rot_dim) {
-      if (e < half) v = v * cosines[e] - sum_splits(in + c + half, nsplit, split_stride) * sines[e];
-      else v = v * cosines[e - half] + sum_splits(in + c - half, nsplit, split_stride) * sines[e - half];
+      if (e < half) v = v * cosines[e] - normed(c + half) * sines[e];
+      else v = v * cosines[e - half] + normed(c - half) * sines[e - half];
     }
-    if (head < nq) q_out[static_cast<size_t>(t) * nq * d + c] = from_float<A>(v);
-    else page[(static_cast<size_t>(head - nq) * page_size + row) * d + e] = from_float<A>(v);
+    if (head < nq) {
+      q_out[static_cast<size_t>(t) * nq * d + c] = from_float<A>(v);
+    } else {
+      page[(static_cast<size_t>(head - nq) * page_size + row) * d + e] = from_float<A>(v);
+      if (options.values_are_keys)
+        page[static_cast<size_t>(nkv) * page_size * d + (static_cast<size_t>(head - nq) * d + e) * page_size + row] =
+            from_float<A>(sum_splits(in + c, nsplit, split_stride));
+    }
   }
 }
 
@@ -187,24 +237,30 @@ using namespace tlie;
 
 // q heads of d | k heads of d | nv value heads of dv (nv = nkv, or fewer when several key heads share a value head:
 // a page then holds the nkv planes of keys and after them nv planes of values); a row of the product is
-// row_width columns long, of which these are the first.  See qkv_place_kernel.
+// row_width columns long, of which these are the first.  See qkv_place_kernel and PlaceOptions (with values_are_keys
+// the product holds no value columns).
 extern "C" int tlie_qkv_place(const void* qkv, int in_dtype, int nsplit, long long split_stride, const int* positions,
                               const int* slot_map, const float* inv_freq, int rot_dim, void* q_out, void* cache,
                               int act_dtype, int tokens, int nq, int nkv, int nv, int d, int dv, int page_size, int row_width,
-                              void* stream) {
+                              const float* q_norm, const float* k_norm, float norm_eps, int values_are_keys, float temp_coef,
+                              float temp_every, void* stream) {
   if (tokens <= 0 || nq <= 0 || nkv < 0 || d <= 0 || dv <= 0 || page_size <= 0 || nsplit < 1) return kBadArgument;
   if (rot_dim < 0 || rot_dim > d || rot_dim % 2 != 0 || (nkv > 0 && (cache == nullptr || slot_map == nullptr))) return kBadArgument;
   if (nv < 0 || nv > nkv || (nkv > 0 && (nv == 0 || nkv % nv != 0))) return kBadArgument;
-  const int width = (nq + nkv) * d + nv * dv;
+  if (values_are_keys && (nv != nkv || dv != d)) return kBadArgument;
+  if ((q_norm != nullptr || k_norm != nullptr) && !(norm_eps > 0.f)) return kBadArgument;
+  if (temp_every < 0.f) return kBadArgument;
+  const int width = (nq + nkv) * d + (values_are_keys ? 0 : nv * dv);
   if (row_width < width) return kBadArgument;
   const int threads = width >= 1024 ? 1024 : (width + 63) / 64 * 64;
-  const size_t lds = static_cast<size_t>(rot_dim) * sizeof(float);
+  const size_t lds = (static_cast<size_t>(rot_dim) + 16) * sizeof(float);
+  const PlaceOptions options{q_norm, k_norm, norm_eps, values_are_keys, temp_coef, temp_every};
   hipStream_t s = (hipStream_t)stream;
 #define TLIE_CASE(DC, D, AC, A)                                                                                \
   if (in_dtype == DC && act_dtype == AC) {                                                                     \
     hipLaunchKernelGGL((qkv_place_kernel<D, A>), dim3(tokens), dim3(threads), lds, s, (const D*)qkv, nsplit,     \
                        (size_t)split_stride, positions, slot_map, inv_freq, rot_dim, (A*)q_out, (A*)cache, nq,  \
-                       nkv, nv, d, dv, page_size, row_width);                                                                \
+                       nkv, nv, d, dv, page_size, row_width, options);                                          \
     return launch_status();                                                                                    \
   }
   TLIE_CASE(kF32, float, kF32, float)

@@ -105,6 +105,9 @@ class DecoderModel:
             residual, pending = self.embedding.forward(ctx.tokens, ctx), None
         if trace is not None:
             trace["embedding"] = residual.float().clone()
+        if self.spec.streams:
+            # a residual of several streams: all start as the embedding's output; the layers work on all of them
+            residual = ops.stream_spread(residual, self.spec.streams)
         for index, run in enumerate(runs):
             next_norm = entry_norm(self.blocks[runs[index + 1].layer]) if index + 1 < len(runs) else self.final_norm
             if trace is not None:
@@ -119,6 +122,10 @@ class DecoderModel:
             pending = self.blocks[run.layer].forward(residual, pending, ctx, bindings[index], next_norm=next_norm)
         if ctx.num_wanted == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)
+        if self.spec.streams:
+            # what goes on is the sum of the streams, with what the last sublayer left joined first
+            _, residual = ops.stream_norm(residual, pending, None, None, 0.0, self.dtype, total=True)
+            pending = None
         if ctx.wants_all_rows:
             lazy = few and self.head.takes_normed_rows(residual.shape[0])
             normed = self.final_norm.add_forward(residual, pending, lazy=lazy)

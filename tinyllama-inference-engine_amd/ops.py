@@ -264,7 +264,8 @@ def attention_generic(q: torch.Tensor, cache: torch.Tensor, block_table: torch.T
                       positions: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
                       window: int | None, scale: float, tiled: bool | int = False, seq_start: torch.Tensor | None = None,
                       min_tokens: int = GENERIC_TILED_MIN_TOKENS, value_dim: int | None = None, chunk: int | None = None,
-                      sink: torch.Tensor | None = None, value_heads: int | None = None, float_out: bool = False) -> torch.Tensor:
+                      sink: torch.Tensor | None = None, value_heads: int | None = None, float_out: bool = False,
+                      softcap: float | None = None) -> torch.Tensor:
     """Causal attention of every token over its sequence's cached keys; any number of tokens per
     sequence.  block_table: [sequences, max_blocks] pages; token_seq[t]: the token's row of it.
     tiled 1 (True): the step's sequences bring several tokens each (consecutive in the step, at
@@ -277,8 +278,11 @@ def attention_generic(q: torch.Tensor, cache: torch.Tensor, block_table: torch.T
     [tokens, nq * value_dim].  chunk: a token sees only the keys of its own chunk of so many positions
     (counted from position 0).  sink: float32 [nq], a number per head whose exponential joins the
     softmax's denominator.  value_heads: fewer value heads than key heads (num_kv_heads / value_heads key heads in
-    a row read one value head; see `_check_cache`).  float_out: the result is float32 whatever q's type."""
+    a row read one value head; see `_check_cache`).  float_out: the result is float32 whatever q's type.
+    softcap: a scaled score s enters the softmax as softcap * tanh(s / softcap)."""
     _device_tensor(q, "q", (torch.float32, torch.bfloat16))
+    if softcap is not None and not float(softcap) > 0.0:
+        raise invalid_argument("attention: a cap of the scores must be positive")
     value_dim = head_dim if value_dim is None else int(value_dim)
     value_heads = num_kv_heads if value_heads is None else int(value_heads)
     if sink is not None:
@@ -315,7 +319,8 @@ def attention_generic(q: torch.Tensor, cache: torch.Tensor, block_table: torch.T
                                             int(window) if window else 0, int(chunk) if chunk else 0, _ptr(sink),
                                             ctypes.c_float(scale), tiled,
                                             _ptr(seq_start if tiled == 2 else None), int(min_tokens),
-                                            num_kv_heads // value_heads, 1 if float_out else 0, _stream()),
+                                            num_kv_heads // value_heads, 1 if float_out else 0,
+                                            ctypes.c_float(float(softcap) if softcap else 0.0), _stream()),
            "attention_generic")
     return out
 
@@ -372,17 +377,33 @@ def norm_add_rmsnorm(residual: torch.Tensor, delta: Product, post_weight: torch.
 
 def qkv_place(qkv: Product, positions: torch.Tensor, slot_map: torch.Tensor | None, inv_freq: torch.Tensor | None,
               rot_dim: int, cache: torch.Tensor | None, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int,
-              act_dtype: torch.dtype, value_heads: int | None = None, extra_cols: int = 0) -> torch.Tensor:
+              act_dtype: torch.dtype, value_heads: int | None = None, extra_cols: int = 0,
+              q_norm: torch.Tensor | None = None, k_norm: torch.Tensor | None = None, norm_eps: float = 0.0,
+              values_are_keys: bool = False, q_temp: tuple[float, float] | None = None) -> torch.Tensor:
     """`rope_cache` for any sizes: value heads of `value_dim` dims (a page is then nkv planes of keys and
     after them nkv planes of transposed values), and num_kv_heads 0 for a layer that reads another
     layer's cache: only its queries [T, nq * d] are rotated and returned, nothing is written.
     value_heads: fewer value heads than key heads (see `_check_cache`).  extra_cols: columns that the product
-    has after q, k and v, which are someone else's to read."""
+    has after q, k and v, which are someone else's to read.
+    q_norm, k_norm (float32 [nq * d], [nkv * d]): all of a token's query columns together, and all of its key columns
+    together, are RMS-normed (norm_eps inside the root) and multiplied by the weight before the rotation.
+    values_are_keys: the product holds no value columns; a key head as projected, before norm and rotation, is also its
+    value head (value_dim = head_dim).  q_temp (coef, every): a query at position p is multiplied by
+    1 + coef * ln(floor((p + 1) / every) + 1)."""
     _check_product(qkv, "qkv")
+    if values_are_keys and (value_dim != head_dim or (value_heads is not None and value_heads != num_kv_heads) or num_kv_heads == 0):
+        raise invalid_shape("qkv_place: values that are the keys have the keys' heads and size")
+    for name, weight, count in (("q_norm", q_norm, num_heads * head_dim), ("k_norm", k_norm, num_kv_heads * head_dim)):
+        if weight is not None:
+            _device_tensor(weight, name, torch.float32)
+            if weight.shape != (count,) or not norm_eps > 0.0:
+                raise invalid_shape(f"qkv_place: {name} needs {count} entries and a positive eps")
+    if q_temp is not None and not float(q_temp[1]) > 0.0:
+        raise invalid_argument("qkv_place: the query temperature's period must be positive")
     _device_tensor(positions, "positions", torch.int32)
     tokens = qkv.rows
     value_heads = num_kv_heads if value_heads is None else int(value_heads)
-    if extra_cols < 0 or qkv.cols != (num_heads + num_kv_heads) * head_dim + value_heads * value_dim + extra_cols:
+    if extra_cols < 0 or qkv.cols != (num_heads + num_kv_heads) * head_dim + (0 if values_are_keys else value_heads * value_dim) + extra_cols:
         raise invalid_shape(f"qkv_place: qkv width {qkv.cols} is not (nq + nkv) * d + nv * dv + {extra_cols}")
     if positions.shape != (tokens,):
         raise invalid_shape("qkv_place: positions need one entry per token")
@@ -403,7 +424,10 @@ def qkv_place(qkv: Product, positions: torch.Tensor, slot_map: torch.Tensor | No
     _check(library().tlie_qkv_place(_ptr(qkv.data), dtype_code(qkv.data.dtype), qkv.nsplit, ctypes.c_longlong(qkv.split_stride),
                                     _ptr(positions), _ptr(slot_map if num_kv_heads > 0 else None), _ptr(inv_freq), rot_dim,
                                     _ptr(q_out), _ptr(cache if num_kv_heads > 0 else None), dtype_code(act_dtype), tokens,
-                                    num_heads, num_kv_heads, value_heads, head_dim, value_dim, page_size, qkv.cols, _stream()),
+                                    num_heads, num_kv_heads, value_heads, head_dim, value_dim, page_size, qkv.cols,
+                                    _ptr(q_norm), _ptr(k_norm), ctypes.c_float(norm_eps), 1 if values_are_keys else 0,
+                                    ctypes.c_float(float(q_temp[0]) if q_temp else 0.0),
+                                    ctypes.c_float(float(q_temp[1]) if q_temp else 0.0), _stream()),
            "qkv_place")
     return q_out
 
@@ -461,7 +485,8 @@ def block_linear(x: torch.Tensor, x_offset: int, x_row: int, x_block: int, weigh
 
 def latent_place(fused: Product, positions: torch.Tensor, slot_map: torch.Tensor, inv_freq: torch.Tensor | None,
                  norm_weight: torch.Tensor, eps: float, cache: torch.Tensor, heads: int, plain: int, rot: int, rank: int,
-                 act_dtype: torch.dtype, wide_values: bool = False, turn: int | None = None) -> tuple[torch.Tensor, torch.Tensor]:
+                 act_dtype: torch.dtype, wide_values: bool = False, turn: int | None = None,
+                 extra_cols: int = 0) -> tuple[torch.Tensor, torch.Tensor]:
     """Latent attention between its first product and the attention kernel.  fused: [T, heads * (plain +
     rot) + rank + rot].  The rank dims are RMS-normed (weight, eps) and written to the cache rows of
     `slot_map` as keys [row][rank + rot] beside the rotated shared key part, and once more, transposed, as
@@ -470,14 +495,14 @@ def latent_place(fused: Product, positions: torch.Tensor, slot_map: torch.Tensor
     wide_values: the value side of a page has rank + rot rows, as many as a key has dims (the cache is then
     [pages, 2, 1, page_size * (rank + rot)], what an attention kernel with one head size reads); its last rot
     rows are never written.  turn: how many of the rot dims are rotated (the first ones; default all), inv_freq
-    then has turn / 2 entries."""
+    then has turn / 2 entries.  extra_cols: columns that the product has after these, which are someone else's to read."""
     _check_product(fused, "fused")
     _device_tensor(positions, "positions", torch.int32)
     _device_tensor(slot_map, "slot_map", torch.int32)
     _device_tensor(cache, "cache", act_dtype)
     _device_tensor(norm_weight, "latent norm weight", (torch.float32, torch.bfloat16))
     tokens = fused.rows
-    if fused.cols != heads * (plain + rot) + rank + rot or norm_weight.shape != (rank,):
+    if extra_cols < 0 or fused.cols != heads * (plain + rot) + rank + rot + extra_cols or norm_weight.shape != (rank,):
         raise invalid_shape(f"latent_place: width {fused.cols} is not heads * (plain + rot) + rank + rot")
     if positions.shape != (tokens,) or slot_map.shape != (tokens,):
         raise invalid_shape("latent_place: positions and slot_map need one entry per token")
@@ -495,7 +520,7 @@ def latent_place(fused: Product, positions: torch.Tensor, slot_map: torch.Tensor
                                        ctypes.c_longlong(fused.split_stride), _ptr(positions), _ptr(slot_map), _ptr(inv_freq),
                                        _ptr(norm_weight), dtype_code(norm_weight.dtype), ctypes.c_float(eps), _ptr(q_plain),
                                        _ptr(q_wide), _ptr(cache), dtype_code(act_dtype), tokens, heads, plain, rot, turn, rank,
-                                       rank + rot if wide_values else rank, page_size, _stream()), "latent_place")
+                                       rank + rot if wide_values else rank, page_size, fused.cols, _stream()), "latent_place")
     return q_plain, q_wide
 
 
@@ -962,9 +987,20 @@ def decay_scan(q: tuple[Product, int], k: tuple[Product, int], v: tuple[Product,
     return out
 
 
-def few_outputs(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None, top: int = 0) -> torch.Tensor:
+ROUTER_SCORES = {"sigmoid": 0, "softmax_of_chosen": 1}
+
+
+def few_outputs(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None, top: int = 0,
+                score: str = "sigmoid", extra: int = 0) -> torch.Tensor:
     """A product with few outputs and float sums: float32 [tokens, outputs] = x . weight^T + bias.  top > 0: as a
-    router: the sigmoids of the sums, of which each token's `top` largest keep their value and the rest become 0."""
+    router: score "sigmoid": the sigmoids of the sums, of which each token's `top` largest keep their value and the rest
+    become 0; score "softmax_of_chosen": each token's `top` largest sums are chosen and keep their softmax over the
+    chosen ones only (at most 64), the rest become 0.  extra: the last `extra` outputs stand outside the choice and become
+    their own sigmoids (gates of something every token uses)."""
+    if score not in ROUTER_SCORES:
+        raise invalid_argument(f"few_outputs: unknown score '{score}'")
+    if extra < 0 or (top == 0 and (extra or score != "sigmoid")):
+        raise invalid_argument("few_outputs: scores and extra outputs go with a router (top > 0)")
     _device_tensor(x, "x", (torch.float32, torch.bfloat16))
     _device_tensor(weight, "weight", (torch.float32, torch.bfloat16))
     if x.dim() != 2 or weight.dim() != 2 or x.shape[1] != weight.shape[1]:
@@ -976,35 +1012,139 @@ def few_outputs(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None
         _device_tensor(bias, "bias", weight.dtype)
         if bias.shape != (outputs,):
             raise invalid_shape("few_outputs: the bias needs one entry per output")
-    if top < 0 or top > outputs:
-        raise invalid_argument("few_outputs: a router picks between 1 and all of its outputs")
+    if top < 0 or top > outputs - extra or (score == "softmax_of_chosen" and top > 64):
+        raise invalid_argument("few_outputs: a router picks between 1 and all of its outputs (a softmax over at most 64)")
     out = torch.empty((x.shape[0], outputs), dtype=torch.float32, device=x.device)
     if x.shape[0] == 0:
         return out
     _check(library().tlie_few_outputs(_ptr(x), dtype_code(x.dtype), _ptr(weight), _ptr(bias), dtype_code(weight.dtype),
-                                      _ptr(out), x.shape[0], x.shape[1], outputs, int(top), _stream()), "few_outputs")
+                                      _ptr(out), x.shape[0], x.shape[1], outputs, int(top), ROUTER_SCORES[score], int(extra),
+                                      _stream()), "few_outputs")
     return out
 
 
-def routed_gate(gate_up: Product, scale: torch.Tensor, block: int, out_dtype: torch.dtype) -> torch.Tensor:
+def routed_gate(gate_up: Product, scale: torch.Tensor, block: int, out_dtype: torch.dtype, weigh: str = "input",
+                shared_scaled: bool = False, gate: str = "silu", alpha: float = 1.0, limit: float = 0.0,
+                shared_limit: float | None = None) -> torch.Tensor:
     """hidden[t, c] = silu(s g) * (s u): g and u side by side in gate_up (g0 u0 g1 u1 ...), s = scale[t, c // block]
     for the columns of the experts (scale: float32 [tokens, experts], 0 for an expert the token does not use) and 1
-    for the columns after them (an expert that every token uses)."""
+    for the columns after them (an expert that every token uses).
+    weigh "output": hidden[t, c] = s * act(g, u), the score weighs what the expert gives (the product that follows is
+    linear); the gate may then be any of `GATES` with its alpha and limit (shared_limit: the limit of the columns after
+    the experts', default the same).  shared_scaled: scale has one column more, which the columns after the experts'
+    take in the place of 1."""
     _check_product(gate_up, "gate_up")
     _device_tensor(scale, "scale", torch.float32)
     if gate_up.cols % 2 != 0:
         raise invalid_shape("routed_gate: gate and up lie side by side, the width must be even")
     rows, inter = gate_up.rows, gate_up.cols // 2
-    if scale.dim() != 2 or scale.shape[0] != rows or block <= 0 or scale.shape[1] * block > inter:
+    if weigh not in ("input", "output") or gate not in GATES or (weigh == "input" and gate != "silu"):
+        raise invalid_argument("routed_gate: a score weighs the input (SiLU gate) or the output (any gate)")
+    if gate == "clamped_swish" and not (limit > 0.0 and (shared_limit is None or shared_limit > 0.0)):
+        raise invalid_argument("routed_gate: the clamped gate needs positive limits")
+    experts = scale.shape[1] - (1 if shared_scaled else 0) if scale.dim() == 2 else -1
+    if scale.dim() != 2 or scale.shape[0] != rows or block <= 0 or experts < 0 or experts * block > inter:
         raise invalid_shape("routed_gate: the scale matrix does not fit the columns")
     out = torch.empty((rows, inter), dtype=out_dtype, device=gate_up.data.device)
     if rows == 0:
         return out
     _check(library().tlie_routed_gate(_ptr(gate_up.data), dtype_code(gate_up.data.dtype), gate_up.nsplit,
-                                      ctypes.c_longlong(gate_up.split_stride), _ptr(scale), scale.shape[1], int(block),
-                                      _ptr(out), dtype_code(out_dtype), rows, inter, _stream()), "routed_gate")
+                                      ctypes.c_longlong(gate_up.split_stride), _ptr(scale), experts, int(block),
+                                      _ptr(out), dtype_code(out_dtype), rows, inter, 1 if weigh == "output" else 0,
+                                      scale.shape[1], 1 if shared_scaled else 0, GATES[gate], ctypes.c_float(alpha),
+                                      ctypes.c_float(limit), ctypes.c_float(limit if shared_limit is None else shared_limit),
+                                      _stream()), "routed_gate")
     return out
 
+
+
+def sigmoid_gate(values: torch.Tensor, pre: Product, col: int) -> torch.Tensor:
+    """values[t, c] *= sigmoid(pre[t, col + c]), in place: a gate on a mixer's heads whose pre-activations are columns
+    of a wider product; the sigmoid and the product are float."""
+    _device_tensor(values, "values", (torch.float32, torch.bfloat16))
+    _check_product(pre, "pre")
+    if values.dim() != 2 or values.shape[0] != pre.rows or col < 0 or col + values.shape[1] > pre.cols:
+        raise invalid_shape(f"sigmoid_gate: columns {col} .. of a product [{pre.rows}, {pre.cols}] do not fit values {list(values.shape)}")
+    if values.shape[0] == 0:
+        return values
+    _check(library().tlie_sigmoid_gate(_ptr(values), dtype_code(values.dtype), _ptr(pre.data), dtype_code(pre.data.dtype), pre.nsplit,
+                                       ctypes.c_longlong(pre.split_stride), int(col), pre.cols, values.shape[0], values.shape[1],
+                                       _stream()), "sigmoid_gate")
+    return values
+
+
+def softcap(x: torch.Tensor, cap: float) -> torch.Tensor:
+    """x <- cap * tanh(x / cap), in place, on floats."""
+    _device_tensor(x, "x", torch.float32)
+    if not cap > 0.0:
+        raise invalid_argument("softcap: the cap must be positive")
+    if x.numel() > 0:
+        _check(library().tlie_softcap(_ptr(x), ctypes.c_longlong(x.numel()), ctypes.c_float(cap), _stream()), "softcap")
+    return x
+
+
+MAX_STREAMS = 8        # the most streams a residual of several may have
+
+
+@dataclass
+class StreamUpdate:
+    """What a residual of several streams still lacks: a sublayer's result and how it joins, `mix` float32 [S, S]
+    ([from, to]) and `write` float32 [S]: x_t <- sum_s mix[s, t] x_s + write[t] * result.  Whoever reads the streams next
+    brings them up to date in the same kernel (`stream_norm`)."""
+    product: Product
+    mix: torch.Tensor
+    write: torch.Tensor
+
+
+def stream_spread(first: torch.Tensor, count: int) -> torch.Tensor:
+    """float32 [count, tokens, hidden]: `count` copies of `first` [tokens, hidden]."""
+    _device_tensor(first, "first", torch.float32)
+    if first.dim() != 2 or not 0 < count <= MAX_STREAMS:
+        raise invalid_shape(f"stream_spread: [tokens, hidden] floats into 1 to {MAX_STREAMS} streams")
+    out = torch.empty((count, *first.shape), dtype=torch.float32, device=first.device)
+    if first.numel() > 0:
+        _check(library().tlie_stream_spread(_ptr(first), _ptr(out), int(count), ctypes.c_longlong(first.numel()), _stream()), "stream_spread")
+    return out
+
+
+def stream_norm(streams: torch.Tensor, update: StreamUpdate | None, read: torch.Tensor | None, weight: torch.Tensor | None,
+                eps: float, out_dtype: torch.dtype, total: bool = False):
+    """Between two sublayers of a residual of several streams (float32 [S, tokens, hidden], changed in place): the
+    streams are brought up to date with `update` (or left, None); then, with `read` (float32 [S]), u = sum_s read[s] x_s is
+    RMS-normed with `weight` and `eps` and returned in `out_dtype`; with `total` the sum of the streams is returned too
+    (float32 [tokens, hidden]).  Returns (normed or None, total or None)."""
+    _device_tensor(streams, "streams", torch.float32)
+    if streams.dim() != 3 or not 0 < streams.shape[0] <= MAX_STREAMS:
+        raise invalid_shape(f"stream_norm: the streams must be [1 to {MAX_STREAMS}, tokens, hidden]")
+    count, tokens, hidden = streams.shape
+    delta = None
+    if update is not None:
+        delta = update.product
+        _check_product(delta, "delta")
+        _device_tensor(update.mix, "mix", torch.float32)
+        _device_tensor(update.write, "write", torch.float32)
+        if (delta.rows, delta.cols) != (tokens, hidden) or update.mix.shape != (count, count) or update.write.shape != (count,):
+            raise invalid_shape("stream_norm: the result, mix [S, S] and write [S] do not fit the streams")
+    out = None
+    if read is not None:
+        _device_tensor(read, "read", torch.float32)
+        _device_tensor(weight, "norm weight", (torch.float32, torch.bfloat16))
+        if read.shape != (count,) or weight.shape != (hidden,):
+            raise invalid_shape("stream_norm: read [S] and the norm's weight [hidden] do not fit the streams")
+        if not eps > 0.0:
+            raise EngineError(ErrorCode.NUMERICAL, "RMSNorm requires a positive epsilon")
+        out = torch.empty((tokens, hidden), dtype=out_dtype, device=streams.device)
+    summed = torch.empty((tokens, hidden), dtype=torch.float32, device=streams.device) if total else None
+    if tokens == 0 or (update is None and read is None and not total):
+        return out, summed
+    _check(library().tlie_stream_norm(_ptr(streams), count, _ptr(delta.data if delta is not None else None),
+                                      dtype_code(delta.data.dtype) if delta is not None else F32, delta.nsplit if delta is not None else 1,
+                                      ctypes.c_longlong(delta.split_stride if delta is not None else 0),
+                                      _ptr(update.mix if update is not None else None), _ptr(update.write if update is not None else None),
+                                      _ptr(read), _ptr(weight), dtype_code(weight.dtype) if weight is not None else F32,
+                                      ctypes.c_float(eps if read is not None else 1.0), _ptr(out), dtype_code(out_dtype) if out is not None else F32,
+                                      _ptr(summed), tokens, hidden, _stream()), "stream_norm")
+    return out, summed
 
 def residual_update(residual: torch.Tensor, first: Product, second: Product | None, mult: float,
                     copy_dtype: torch.dtype | None = None) -> torch.Tensor | None:

@@ -34,11 +34,17 @@ class Attention(Mixer):
       reads_other_cache  the layer has no key and value projections: it reads the cache its run names
       cache_window       how long the cache keeps a position (default: window, or chunk); the owner of a
                          cache that other layers read names the longest reach among them (None: for good)
-      names              the tensors' names after the prefix, by role (q, k, v, o, q_bias .. o_bias, sink)
+      softcap            c: a scaled score s enters the softmax as c * tanh(s / c)
+      q_temp             (coef, every): the query at position p is multiplied by 1 + coef * ln(floor((p + 1) / every) + 1)
+      values_are_keys    there is no value projection: a key head as projected, before any norm and rotation, is also
+                         its value head
+      qk_norm            "whole": all of a token's query columns together, and all of its key columns together, are
+                         RMS-normed (norm_eps) with a weight of that many entries (q_norm, k_norm), before the rotation
+      names              the tensors' names after the prefix, by role (q, k, v, o, q_bias .. o_bias, sink, q_norm, k_norm)
     Tensors: `<prefix>{q,k,v,o}_proj.weight` (and `.bias` when bias) unless `names` says otherwise."""
     NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
              "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "o_bias": "o_proj.bias",
-             "sink": "sinks"}
+             "sink": "sinks", "q_norm": "q_norm.weight", "k_norm": "k_norm.weight"}
 
     def __init__(self, spec: PartSpec, dtype, device):
         super().__init__(spec, dtype, device)
@@ -69,11 +75,26 @@ class Attention(Mixer):
             raise invalid_config("attention: a chunk must be a positive count of positions")
         if not (self.scale > 0.0 and math.isfinite(self.scale)):
             raise invalid_config("attention: the scale of the scores must be positive")
+        self.softcap = float(spec["softcap"]) if spec.get("softcap") is not None else None
+        self.q_temp = tuple(float(number) for number in spec["q_temp"]) if spec.get("q_temp") is not None else None
+        self.values_are_keys = bool(spec.get("values_are_keys", False))
+        self.qk_norm = spec.get("qk_norm")
+        self.norm_eps = float(spec.get("norm_eps", 0.0))
+        if self.softcap is not None and not self.softcap > 0.0:
+            raise invalid_config("attention: a cap of the scores must be positive")
+        if self.q_temp is not None and (len(self.q_temp) != 2 or not self.q_temp[1] > 0.0):
+            raise invalid_config("attention: a query temperature is (coef, every) with a positive period")
+        if self.values_are_keys and (self.dv != self.d or self.reads_other_cache or self.bias):
+            raise invalid_config("attention: values that are the keys have the keys' size, and the layer its own keys and no biases")
+        if self.qk_norm not in (None, "whole") or (self.qk_norm is not None and (not self.norm_eps > 0.0 or self.reads_other_cache)):
+            raise invalid_config("attention: qk_norm is \"whole\" (with a positive norm_eps, on a layer with keys of its own) or absent")
         # what the kernels that are fused for the plain case (one head size, no sink, no chunks, own keys
-        # and values) do not take goes through the kernels for any sizes
-        self.general = self.dv != self.d or self.has_sink or self.chunk is not None or self.reads_other_cache
+        # and values, scores as they are) do not take goes through the kernels for any sizes
+        self.placed = self.q_temp is not None or self.values_are_keys or self.qk_norm is not None   # options of the placement kernel alone
+        self.general = (self.dv != self.d or self.has_sink or self.chunk is not None or self.reads_other_cache
+                        or self.softcap is not None or self.placed)
         self.names = {**self.NAMES, **dict(spec.get("names") or {})}
-        self.qkv = self.o = self.sink = None
+        self.qkv = self.o = self.sink = self.q_norm = self.k_norm = None
 
     @classmethod
     def tensor_specs(cls, spec, prefix):
@@ -83,9 +104,13 @@ class Attention(Mixer):
         nq, nkv = int(spec["num_heads"]), int(spec["num_kv_heads"])
         shapes = [("q", (nq * d, hidden))]
         if not spec.get("reads_other_cache", False):
-            shapes += [("k", (nkv * d, hidden)), ("v", (nkv * dv, hidden))]
+            shapes.append(("k", (nkv * d, hidden)))
+            if not spec.get("values_are_keys", False):
+                shapes.append(("v", (nkv * dv, hidden)))
         shapes.append(("o", (hidden, nq * dv)))
         specs = [TensorSpec(prefix + names[role], shape) for role, shape in shapes]
+        if spec.get("qk_norm") is not None:
+            specs += [TensorSpec(prefix + names["q_norm"], (nq * d,), init="norm"), TensorSpec(prefix + names["k_norm"], (nkv * d,), init="norm")]
         if spec.get("bias", False):
             specs += [TensorSpec(prefix + names[role + "_bias"], (shape[0],)) for role, shape in shapes]
         if spec.get("sink", False):
@@ -101,7 +126,7 @@ class Attention(Mixer):
         self.paired = table is not None and not self.general
         order = ops.paired_rows(self.nq, self.nkv, self.d, table[1]).to(self.device) if self.paired else None
         names = self.names
-        roles = ("q",) if self.reads_other_cache else ("q", "k", "v")
+        roles = ("q",) if self.reads_other_cache else (("q", "k") if self.values_are_keys else ("q", "k", "v"))
 
         def cat(suffix):
             joined = torch.cat([weights[prefix + names[role + suffix]] for role in roles], dim=0)
@@ -112,6 +137,9 @@ class Attention(Mixer):
                         self.dtype, keep=keep)
         if self.has_sink:
             self.sink = keep(weights[prefix + names["sink"]].float().contiguous())     # (it enters the softmax, which is float)
+        if self.qk_norm is not None:                       # (norms are float)
+            self.q_norm = keep(weights[prefix + names["q_norm"]].float().contiguous())
+            self.k_norm = keep(weights[prefix + names["k_norm"]].float().contiguous())
 
     @property
     def graph_safe(self) -> bool:
@@ -151,15 +179,17 @@ class Attention(Mixer):
         inv_freq, rot_dim = table if table is not None else (None, 0)
         writes = binding.writes and not self.reads_other_cache
         q = None
-        if (table is None and self.dv == self.d and self.d % 2 == 0 and not self.reads_other_cache
+        if (table is None and self.dv == self.d and self.d % 2 == 0 and not self.reads_other_cache and not self.placed
                 and self.qkv.takes_rows(x.shape[0])):
             # a step of few rows, one head size, own keys and values: the product places q and writes the cache itself
             q = self.qkv(x, rope=ops.RopeTarget(ctx.positions, pages.slot_map if writes else ctx.no_slots, None, 0, binding.cache,
                                                 self.nq, self.nkv, self.d))
         if q is None or isinstance(q, ops.Product):
             q = ops.qkv_place(ops.as_product(q if q is not None else self.qkv(x)), ctx.positions, pages.slot_map if writes else ctx.no_slots, inv_freq,
-                          rot_dim, binding.cache, self.nq, 0 if self.reads_other_cache else self.nkv, self.d, self.dv, self.dtype)
-        if self.dv == self.d and ops.attention_mfma_takes(self.dtype, self.d, binding.cache.shape[3] // self.d):
+                          rot_dim, binding.cache, self.nq, 0 if self.reads_other_cache else self.nkv, self.d, self.dv, self.dtype,
+                          q_norm=self.q_norm, k_norm=self.k_norm, norm_eps=self.norm_eps, values_are_keys=self.values_are_keys,
+                          q_temp=self.q_temp)
+        if self.dv == self.d and self.softcap is None and ops.attention_mfma_takes(self.dtype, self.d, binding.cache.shape[3] // self.d):
             # bfloat16, one head size: the kernel on the matrix cores (scores, softmax and sink float)
             tiles, col_tiles, nsplit, split_len, waves, shared = ops.attention_plan(ctx, self.nq // self.nkv, self.nkv, self.d)
             attended = ops.attention_mfma(q, binding.cache, pages.block_table, tiles, ctx.positions, self.nq, self.nkv, self.d,
@@ -168,7 +198,8 @@ class Attention(Mixer):
         else:
             attended = ops.attention_generic(q, binding.cache, pages.block_table, ctx.token_seq, ctx.positions, self.nq, self.nkv,
                                              self.d, self.window, self.scale, tiled=ops.attention_generic_plan(ctx, self.d, self.dv),
-                                             seq_start=ctx.seq_start, value_dim=self.dv, chunk=self.chunk, sink=self.sink)
+                                             seq_start=ctx.seq_start, value_dim=self.dv, chunk=self.chunk, sink=self.sink,
+                                             softcap=self.softcap)
         return self.o(attended)
 
     def forward(self, x, ctx, binding: Binding, into=None):

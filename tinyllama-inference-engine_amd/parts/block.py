@@ -362,3 +362,105 @@ class ParallelBlock:
         ops.norm_add_rmsnorm(residual, waiting.product, waiting.weight, waiting.eps, None, waiting.eps, self.dtype)
         keep("output", residual)
         return None
+
+
+@register("block", "hyper_connections")
+class HyperConnectionBlock:
+    """A pre-norm layer on a residual of S streams x_1 .. x_S (`LayerSpec.streams`; float32 [S, tokens, hidden]).  For the
+    mixer and then, if the layer has one, the feed-forward, each with three tensors of its own (`in` [S], `mix` [S, S],
+    `out` [S]):
+        u = sum_s in[s] x_s;   y = sublayer(norm(u));   x_t <- sum_s mix[s, t] x_s + out[t] * y   (all streams at once)
+    The block does not bring the streams up to date itself: a result waits as an `ops.StreamUpdate`, and the kernel that
+    forms the next sublayer's u (this block's, the next block's, or the model's sum over the streams at the end) applies
+    it first.  The norms must be RMS norms that hand out their weight (`lazy_params`)."""
+
+    def __init__(self, layer: LayerSpec, dtype, device):
+        from ..errors import invalid_config
+        self.layer = layer
+        self.dtype = dtype
+        self.streams = int(layer.streams)
+        if not 0 < self.streams <= ops.MAX_STREAMS:
+            raise invalid_config(f"a hyper_connections layer works on 1 to {ops.MAX_STREAMS} streams")
+        self.mixer_norm = lookup("norm", layer.mixer_norm.kind)(layer.mixer_norm, dtype, device)
+        self.mixer = lookup("mixer", layer.mixer.kind)(layer.mixer, dtype, device)
+        self.feed_forward = self.feed_forward_norm = None
+        if layer.feed_forward is not None:
+            self.feed_forward_norm = lookup("norm", layer.feed_forward_norm.kind)(layer.feed_forward_norm, dtype, device)
+            self.feed_forward = lookup("feed_forward", layer.feed_forward.kind)(layer.feed_forward, dtype, device)
+        for norm in (self.mixer_norm, self.feed_forward_norm):
+            if norm is not None and norm.lazy_params() is None and not hasattr(norm, "weight"):
+                raise invalid_config("a hyper_connections layer's norms must be RMS norms")
+        self.mixer_streams = self.feed_forward_streams = None      # each (in, mix, out) as float tensors
+
+    @classmethod
+    def _parts(cls, layer: LayerSpec):
+        parts = [("mixer_norm", "norm"), ("mixer", "mixer")]
+        if layer.feed_forward is not None:
+            parts += [("feed_forward_norm", "norm"), ("feed_forward", "feed_forward")]
+        return parts
+
+    @classmethod
+    def _stream_places(cls, layer: LayerSpec):
+        places = [("mixer_streams", layer.prefix + layer.mixer_streams_place)]
+        if layer.feed_forward is not None:
+            places.append(("feed_forward_streams", layer.prefix + layer.feed_forward_streams_place))
+        return places
+
+    @classmethod
+    def tensor_specs(cls, layer: LayerSpec):
+        from ..config.spec import TensorSpec
+        specs = []
+        for attribute, table in cls._parts(layer):
+            part_spec = getattr(layer, attribute)
+            specs += lookup(table, part_spec.kind).tensor_specs(part_spec, layer.prefix + getattr(layer, attribute + "_place"))
+        count = int(layer.streams)
+        for _, place in cls._stream_places(layer):
+            specs += [TensorSpec(place + "in", (count,), init="share"), TensorSpec(place + "out", (count,), init="norm"),
+                      TensorSpec(place + "mix", (count, count), init="near_identity")]
+        return specs
+
+    def load(self, weights):
+        from ..weights.arena import keep_in
+        for attribute, _ in self._parts(self.layer):
+            getattr(self, attribute).load(weights, self.layer.prefix + getattr(self.layer, attribute + "_place"))
+        for attribute, place in self._stream_places(self.layer):
+            # (the residual's arithmetic is float: so are these few numbers)
+            setattr(self, attribute, tuple(keep_in(weights, weights[place + name].float().contiguous()) for name in ("in", "mix", "out")))
+
+    def entry_norm(self):
+        return None
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(getattr(getattr(self, attribute), "graph_safe", False) for attribute, _ in self._parts(self.layer))
+
+    def forward(self, streams, pending, ctx, binding, next_norm=None):
+        """`streams`: float32 [S, tokens, hidden]; `pending`: an `ops.StreamUpdate` that the streams still lack, or None.
+        A step that keeps a trace leaves, under `ctx.trace_prefix`, "input_norm", "attention_output", with a feed-forward
+        "post_attention_norm" and "mlp_output", and "output", the sum of the streams after the layer (the block then
+        brings the streams up to date itself and hands on nothing)."""
+        trace = getattr(ctx, "trace", None)
+        if streams.dim() != 3 or streams.shape[0] != self.streams:
+            raise ops.invalid_shape(f"a hyper_connections layer works on [{self.streams}, tokens, hidden] streams, not {list(streams.shape)}")
+        if pending is not None and not isinstance(pending, ops.StreamUpdate):
+            raise ops.invalid_argument("what a residual of several streams still lacks must say how it joins them")
+
+        def keep(name, tensor):
+            if trace is not None:
+                trace[ctx.trace_prefix + name] = tensor.float().clone()
+        sublayers = [(self.mixer_norm, self.mixer_streams, lambda x: self.mixer.forward(x, ctx, binding), "input_norm", "attention_output")]
+        if self.feed_forward is not None:
+            sublayers.append((self.feed_forward_norm, self.feed_forward_streams, lambda x: self.feed_forward.forward(x, ctx),
+                              "post_attention_norm", "mlp_output"))
+        for norm, (read, mix, write), run, normed_name, result_name in sublayers:
+            normed, _ = ops.stream_norm(streams, pending, read, norm.weight, norm.eps, self.dtype)
+            keep(normed_name, normed)
+            result = as_product(run(normed))
+            if trace is not None:
+                keep(result_name, result.dense(torch.float32))
+            pending = ops.StreamUpdate(result, mix, write)
+        if trace is None:
+            return pending
+        _, total = ops.stream_norm(streams, pending, None, None, 0.0, self.dtype, total=True)
+        keep("output", total)
+        return None

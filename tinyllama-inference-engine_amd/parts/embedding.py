@@ -69,11 +69,14 @@ class LMHead(Part):
     def __init__(self, spec: PartSpec, dtype, device):
         """spec: vocab_size, hidden_size, tied (the head's matrix is the embedding's table), and, when
         tied, optionally tied_to: that table's full name (default: the reference's); optionally scale, a factor
-        of the logits (applied to the float sums)."""
+        of the logits (applied to the float sums), and softcap c: the logits leave as c * tanh(logits / c)."""
         super().__init__(spec, dtype, device)
         self.tied = bool(spec.get("tied", False))
         self.tied_to = spec.get("tied_to") or TokenEmbedding.NAME
         self.scale = float(spec.get("scale", 1.0))       # what the logits are multiplied by
+        self.softcap = float(spec["softcap"]) if spec.get("softcap") is not None else None
+        if self.softcap is not None and not self.softcap > 0.0:
+            raise ops.invalid_argument("lm_head: a cap of the logits must be positive")
         self.linear = None
 
     @classmethod
@@ -91,4 +94,6 @@ class LMHead(Part):
 
     def forward(self, normed) -> torch.Tensor:
         logits = self.linear(normed, out_dtype=torch.float32, whole=True).dense(torch.float32)
-        return logits if self.scale == 1.0 else logits.mul_(self.scale)
+        if self.scale != 1.0:
+            logits = logits.mul_(self.scale)
+        return logits if self.softcap is None else ops.softcap(logits.contiguous(), self.softcap)

@@ -38,12 +38,16 @@ class LatentAttention(Mixer):
     ones), value_dim, rank (of the latent vector), scale, norm_eps (of the latent vector's norm), sink (a
     learned number per head in the softmax's denominator), position (a rotation table over the first dims of the
     rot_dim part: all of them, or fewer, the rest then pass unchanged),
+    window (a token sees itself and the window - 1 positions before it; absent: all), output_gate (the heads' results are
+    multiplied by sigmoid(W_gate h), h the mixer's input, before the output projection),
     names (the tensors' names after the prefix, by role).
     Tensors: q [H * (head_dim + rot_dim), hidden], down [rank + rot_dim, hidden], down_norm [rank],
-    up_keys [H * head_dim, rank], up_values [H * value_dim, rank], o [hidden, H * value_dim], sink [H]."""
+    up_keys [H * head_dim, rank], up_values [H * value_dim, rank], o [hidden, H * value_dim], sink [H],
+    gate [H * value_dim, hidden]."""
     graph_safe = True
     NAMES = {"q": "q_proj.weight", "down": "kv_a_proj.weight", "down_norm": "kv_a_layernorm.weight",
-             "up_keys": "k_b_proj.weight", "up_values": "v_b_proj.weight", "o": "o_proj.weight", "sink": "sinks"}
+             "up_keys": "k_b_proj.weight", "up_values": "v_b_proj.weight", "o": "o_proj.weight", "sink": "sinks",
+             "gate": "gate_proj.weight"}
 
     def __init__(self, spec: PartSpec, dtype, device):
         super().__init__(spec, dtype, device)
@@ -56,6 +60,10 @@ class LatentAttention(Mixer):
         self.scale = float(spec.get("scale") or 1.0 / math.sqrt(float(self.plain + self.rot)))
         self.norm_eps = float(spec["norm_eps"])
         self.has_sink = bool(spec.get("sink", False))
+        self.window = int(spec["window"]) if spec.get("window") is not None else None
+        self.output_gate = bool(spec.get("output_gate", False))
+        if self.window is not None and self.window <= 0:
+            raise invalid_config("latent_attention: a window must be a positive count of positions")
         if min(self.heads, self.plain, self.dv, self.rank) <= 0 or self.rot < 0:
             raise invalid_config("latent_attention: sizes must be positive")
         if self.rank > ops.ATTENTION_MAX_HEAD_DIM:
@@ -87,12 +95,17 @@ class LatentAttention(Mixer):
                  TensorSpec(prefix + names["o"], (hidden, heads * dv))]
         if spec.get("sink", False):
             specs.append(TensorSpec(prefix + names["sink"], (heads,)))
+        if spec.get("output_gate", False):
+            specs.append(TensorSpec(prefix + names["gate"], (heads * dv, hidden)))
         return specs
 
     def load(self, weights, prefix):
         names, keep = self.names, partial(keep_in, weights)
-        # one product for the queries and the down projection
-        self.first = Linear(torch.cat([weights[prefix + names["q"]], weights[prefix + names["down"]]], dim=0), None, self.dtype, keep=keep)
+        # one product for the queries and the down projection (and the gate of the heads' results)
+        first = [weights[prefix + names["q"]], weights[prefix + names["down"]]]
+        if self.output_gate:
+            first.append(weights[prefix + names["gate"]])
+        self.first = Linear(torch.cat(first, dim=0), None, self.dtype, keep=keep)
         self.down_norm = keep(weights[prefix + names["down_norm"]].contiguous())
         # per head, as the block-diagonal product wants them, [inner, outer]: a head's query goes to the latent
         # space through W_uk^T (W_uk is [plain, rank] per head: already [inner, outer]); its attended latent
@@ -112,8 +125,8 @@ class LatentAttention(Mixer):
         """One key head of rank + rot dims, [row][dim], then its value dims transposed, [dim][row]: rank of them, or
         with wide values as many as a key has."""
         if self.wide_values:
-            return CacheNeed((2, 1), self.rank + self.rot, None)
-        return CacheNeed((1,), 2 * self.rank + self.rot, None)
+            return CacheNeed((2, 1), self.rank + self.rot, self.window)
+        return CacheNeed((1,), 2 * self.rank + self.rot, self.window)
 
     def forward(self, x, ctx, binding: Binding, into=None):
         pages = ctx.groups[binding.group]
@@ -122,20 +135,23 @@ class LatentAttention(Mixer):
         tokens = fused.rows
         q_plain, q_wide = ops.latent_place(fused, ctx.positions, pages.slot_map if binding.writes else ctx.no_slots, self.inv_freq,
                                            self.down_norm, self.norm_eps, binding.cache, self.heads, self.plain, self.rot,
-                                           self.rank, self.dtype, wide_values=self.wide_values, turn=self.turn)
+                                           self.rank, self.dtype, wide_values=self.wide_values, turn=self.turn,
+                                           extra_cols=self.heads * self.dv if self.output_gate else 0)
         ops.block_linear(q_plain, 0, self.heads * self.plain, self.plain, self.up_keys, None,
                          q_wide, 0, self.heads * key, key, tokens, weight=self.up_keys_rows)
         value_dim = key if self.wide_values else self.rank
         if self.wide_values and ops.attention_mfma_takes(self.dtype, key, binding.cache.shape[-1] // key):
             tiles, col_tiles, nsplit, split_len, waves, shared = ops.attention_plan(ctx, self.heads, 1, key)
             attended = ops.attention_mfma(q_wide, binding.cache, pages.block_table, tiles, ctx.positions, self.heads, 1, key,
-                                          None, self.scale, nsplit, split_len, col_tiles, waves, shared, sink=self.sink)
+                                          self.window, self.scale, nsplit, split_len, col_tiles, waves, shared, sink=self.sink)
         else:
             attended = ops.attention_generic(q_wide, binding.cache, pages.block_table, ctx.token_seq, ctx.positions, self.heads, 1,
-                                             key, None, self.scale, tiled=ops.attention_generic_plan(ctx, key, value_dim),
+                                             key, self.window, self.scale, tiled=ops.attention_generic_plan(ctx, key, value_dim),
                                              seq_start=ctx.seq_start, value_dim=value_dim, sink=self.sink)
         # (of every head's attended vector the first rank dims: with wide values the rest are zeros)
         values = torch.empty((tokens, self.heads * self.dv), dtype=self.dtype, device=attended.device)
         ops.block_linear(attended, 0, self.heads * value_dim, value_dim, self.up_values_t, None,
                          values, 0, self.heads * self.dv, self.dv, tokens, weight=self.up_values_rows)
+        if self.output_gate:
+            ops.sigmoid_gate(values, fused, fused.cols - self.heads * self.dv)
         return self.o(values)

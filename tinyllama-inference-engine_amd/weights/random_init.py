@@ -53,6 +53,10 @@ def _draw(spec: TensorSpec, seed: int, std: float, norm_std: float, dtype: torch
         # the weights of a sum of which the last summand is the main one
         values = values * 0.2
         values[..., -1] += 1.0
+    elif spec.init == "near_identity":
+        values = values * 0.15 + torch.eye(spec.shape[-1], device=device)
+    elif spec.init == "share":
+        values = (1.0 + values * 0.3) / spec.shape[-1]
     else:
         raise ValueError(f"unknown init '{spec.init}' for {spec.name}")
     return values.to(dtype)
