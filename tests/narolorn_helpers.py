@@ -90,8 +90,9 @@ DTYPES = ["float32", "bfloat16"]
 # a row's largest error relative to the row's largest value, against float64 on the same stored weights
 TOLERANCE = {"float32": 3e-5, "bfloat16": 4e-2}
 # two cuts of the same request through the same engine (in bfloat16 a step of few rows takes other product kernels
-# than a step of many, whose results are rounded to bfloat16 where the others' stay float partial sums)
-CUT_TOLERANCE = {"float32": 2e-6, "bfloat16": 4e-2}
+# than a step of many, whose results are rounded to bfloat16 where the others' stay float partial sums: two results that
+# each lie within 4e-2 of the plain one may lie further from each other)
+CUT_TOLERANCE = {"float32": 2e-6, "bfloat16": 6e-2}
 
 
 def make_model(folder, raw_config, seed, std=0.08, norm_std=0.1):

@@ -139,10 +139,22 @@ def router_choice(z, top):
     return chosen, torch.softmax(values, dim=-1)
 
 
-def mixture(mlp, w, prefix, h):
+def router_margin(z, top):
+    """How far each token's choice is from another one: the gap between its `top`-th and its next logit ([T]; infinite
+    when all experts are chosen)."""
+    if top >= z.shape[-1]:
+        return torch.full(z.shape[:-1], math.inf, dtype=z.dtype)
+    ordered = torch.sort(z, dim=-1, descending=True).values
+    return ordered[..., top - 1] - ordered[..., top]
+
+
+def mixture(mlp, w, prefix, h, margins=None):
+    """margins: a list that takes, per call, every token's `router_margin`."""
     experts, top = int(mlp["router"]["experts"]), int(mlp["router"]["top"])
     z = h @ w[prefix + "router"].T + w[prefix + "router.b"]
     chosen, weights = router_choice(z, top)
+    if margins is not None:
+        margins.append(router_margin(z, top))
     out = torch.zeros_like(h)
     for e in range(experts):
         y = expert(w, f"{prefix}e{e}.", h, float(mlp["expert"]["limit"]))
@@ -173,7 +185,8 @@ def hyper_sublayer(streams, w, prefix, sublayer):
     return torch.einsum("sr,std->rtd", w[prefix + "mix"], streams) + w[prefix + "out"][:, None, None] * y[None]
 
 
-def forward(config, weights, tokens):
+def forward(config, weights, tokens, margins=None):
+    """margins: a list that takes every router's margins, one tensor [T] per feed-forward that runs."""
     w = weights
     eps = float(config["norm"]["eps"])
     tokens = torch.as_tensor(tokens, dtype=torch.long)
@@ -190,7 +203,7 @@ def forward(config, weights, tokens):
             return MIXERS[layer["type"]](layer["mixer"], w, prefix + "mix.", rms_norm(u, w[prefix + "norm1"], eps), positions, eps)
 
         def feed(u, layer=layer, prefix=prefix):
-            return mixture(layer["mlp"], w, prefix + "mlp.", rms_norm(u, w[prefix + "norm2"], eps))
+            return mixture(layer["mlp"], w, prefix + "mlp.", rms_norm(u, w[prefix + "norm2"], eps), margins)
         if streams is not None:
             streams = hyper_sublayer(streams, w, prefix + "hc1.", mix)
             if layer.get("mlp") is not None:

@@ -149,6 +149,6 @@ class TensorSpec:
     that the file gives and no configuration names (random weights draw `free_extent` there)."""
     name: str
     shape: tuple[int, ...]
-    init: str = "normal"        # how random weights draw it: "normal", "norm" (around 1), "offset" (a norm's weight stored around 0), "zeros", "forget_bias" (between 3 and 6), "fraction" (between 0 and 1), "mix" (weights of a sum: the last near 1, the others near 0), "near_identity" (a square matrix: 1 on the diagonal, small elsewhere), "share" (numbers around 1 / count)
+    init: str = "normal"        # how random weights draw it: "normal", "norm" (around 1), "offset" (a norm's weight stored around 0), "zeros", "forget_bias" (between 3 and 6), "fraction" (between 0 and 1), "mix" (weights of a sum: the last near 1, the others near 0), "near_identity" (a square matrix: 1 on the diagonal, small elsewhere), "share" (numbers around 1 / count), "spread" (of order 1 whatever the scale of the rest)
     free_extent: int = 16
     optional: bool = False       # absent is no error, present it is checked and not read (a tied head's matrix that some files still carry)

@@ -96,8 +96,9 @@ constexpr int attention_max_waves(int dt, int ct) {
 // longer than what a wave can issue meanwhile), so for head sizes up to 64 the compiler is asked to
 // stay within the registers of 4 waves a SIMD with one column group and 3 with two, where it would
 // take those of 3 and 2 (a prompt of 2048 tokens 53 -> 51 us, of 4096 158 -> 150).
-// EXTRA: the kernel also takes chunks of positions and a sink; without it `chunk` and `sink` are not looked
-// at, and the code is the plain causal (or windowed) kernel's, instruction for instruction (the variant that
+// EXTRA: the kernel also takes chunks of positions, a sink and capped scores (cap_pre > 0: a score s becomes
+// tanh(s * cap_pre) before the mask, cap_pre = scale / cap, and scale_log2 is then cap * log2(e)); without it `chunk`,
+// `sink` and `cap_pre` are not looked at, and the code is the plain causal (or windowed) kernel's, instruction for instruction (the variant that
 // shares keys through LDS is compiled to a tight register budget, which the additions do not fit).
 template <int DT, int CT, bool SHARED, bool EXTRA>
 __global__ void __launch_bounds__(SHARED ? 512 : 64 * attention_max_waves(DT, CT), (SHARED && DT <= 4 && !EXTRA) ? (CT == 1 ? 4 : 3) : 1)
@@ -105,7 +106,7 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
                       const int* __restrict__ block_table, int max_blocks, const int4* __restrict__ tiles,
                       const int* __restrict__ positions, uint16_t* __restrict__ out, float* __restrict__ part_o,
                       float* __restrict__ part_ml, int nsplit, int split_len, int nq, int nkv, int page_size,
-                      int window, int chunk, const float* __restrict__ sink, float scale_log2, int round_size, int plane_map) {
+                      int window, int chunk, const float* __restrict__ sink, float scale_log2, int round_size, int plane_map, float cap_pre) {
   constexpr int D = DT * 16;
   // the first key that the token at position p sees: the window's edge, or the start of the token's own
   // chunk of positions (chunks are counted from position 0), whichever is later; 0 without either
@@ -304,6 +305,16 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
         for (int ks = 0; ks < KS; ++ks)
           s[ct][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(block.k[t][ks].v, qreg[ct][ks].v, s[ct][t], 0, 0, 0);
       }
+    if (EXTRA && cap_pre > 0.f) {
+      // capped scores: tanh(x) = 1 - 2 / (exp(2x) + 1), in base 2; +-1 at the ends, where the exponential is inf or 0
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            s[ct][t][j] = 1.f - 2.f * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(s[ct][t][j] * (cap_pre * 2.8853900817779268f)) + 1.f);
+    }
     // ---- mask; each lane's maximum over its 8 keys of a column (the scale goes into the exponent's
     // multiply-add): s[ct][t][j] is key kb + t*16 + grp*4 + j of the column -------------------------
     float lane_max[CT];
@@ -707,19 +718,21 @@ template <int DT, int CT, bool SHARED = false>
 static int launch_attention(const void* q, const void* cache, const int* block_table, int max_blocks, const void* tiles,
                             int num_tiles, const int* positions, void* out, float* part_o, float* part_ml, int nsplit,
                             int split_len, int nq, int nkv, int page_size, int window, int chunk, const float* sink, float scale,
-                            int waves, hipStream_t stream, int plane_map) {
-  const float scale_log2 = scale * 1.4426950408889634f;
+                            int waves, hipStream_t stream, int plane_map, float softcap) {
+  // (capped scores: the kernel forms tanh(score * scale / cap), and the cap takes the scale's place in the exponent)
+  const float scale_log2 = (softcap > 0.f ? softcap : scale) * 1.4426950408889634f;
+  const float cap_pre = softcap > 0.f ? scale / softcap : 0.f;
   // LDS for merging the waves: their maxima and sums, and half as many slots as waves for the results
   const size_t lds = !SHARED && waves > 1 ? (static_cast<size_t>(waves) * CT * 32 + static_cast<size_t>(waves / 2) * CT * DT * 256) * sizeof(float) : 0;
   if (lds > 64 * 1024) return kBadArgument;
-  if (chunk > 0 || sink != nullptr || plane_map != 0)
+  if (chunk > 0 || sink != nullptr || plane_map != 0 || softcap > 0.f)
     hipLaunchKernelGGL((attention_mfma_kernel<DT, CT, SHARED, true>), dim3(num_tiles, nkv, nsplit), dim3(64 * waves), lds, stream, (const uint16_t*)q,
                        (const uint16_t*)cache, block_table, max_blocks, (const int4*)tiles, positions, (uint16_t*)out, part_o,
-                       part_ml, nsplit, split_len, nq, nkv, page_size, window, chunk, sink, scale_log2, compute_units(), plane_map);
+                       part_ml, nsplit, split_len, nq, nkv, page_size, window, chunk, sink, scale_log2, compute_units(), plane_map, cap_pre);
   else
     hipLaunchKernelGGL((attention_mfma_kernel<DT, CT, SHARED, false>), dim3(num_tiles, nkv, nsplit), dim3(64 * waves), lds, stream, (const uint16_t*)q,
                        (const uint16_t*)cache, block_table, max_blocks, (const int4*)tiles, positions, (uint16_t*)out, part_o,
-                       part_ml, nsplit, split_len, nq, nkv, page_size, window, 0, nullptr, scale_log2, compute_units(), 0);
+                       part_ml, nsplit, split_len, nq, nkv, page_size, window, 0, nullptr, scale_log2, compute_units(), 0, 0.f);
   return launch_status();
 }
 
@@ -741,8 +754,8 @@ static int attention_entry(const void* q, const void* cache, const int* block_ta
                            const void* tiles, int num_tiles, int col_tiles, const int* positions, void* out,
                            float* part_o, float* part_ml, int nsplit, int split_len, int tokens, int nq, int nkv,
                            int d, int page_size, int window, int chunk, const float* sink, float scale, int waves, int shared,
-                           void* stream, int plane_map = 0) {
-  if (chunk < 0) return kBadArgument;
+                           void* stream, int plane_map = 0, float softcap = 0.f) {
+  if (chunk < 0 || softcap < 0.f) return kBadArgument;
   if (plane_map != 0) {
     const int kdiv = plane_map & 255, vgroup = (plane_map >> 8) & 255, vmod = (plane_map >> 16) & 255;
     if (kdiv <= 0 || vgroup <= 0 || vmod <= 0 || vmod > vgroup || nkv % kdiv != 0 || nkv % vgroup != 0 || (plane_map >> 25) != 0)
@@ -764,7 +777,7 @@ static int attention_entry(const void* q, const void* cache, const int* block_ta
   hipStream_t s = (hipStream_t)stream;
   int status = kBadArgument;
 #define TLIE_ARGS q, cache, block_table, max_blocks, tiles, num_tiles, positions, out, part_o, part_ml, nsplit, split_len, nq, \
-                  nkv, page_size, window, chunk, sink, scale, waves, s, plane_map
+                  nkv, page_size, window, chunk, sink, scale, waves, s, plane_map, softcap
 #define TLIE_CASE(DT)                                        \
   case DT:                                                   \
     status = launch_attention<DT, 1>(TLIE_ARGS);             \
@@ -818,6 +831,16 @@ extern "C" int tlie_attention_mfma(const void* q, const void* cache, const int* 
   // sink (or null): float [nq], a number per head whose exponential joins the softmax's denominator
   return attention_entry(q, cache, block_table, max_blocks, tiles, num_tiles, col_tiles, positions, out, part_o, part_ml, nsplit,
                          split_len, tokens, nq, nkv, d, page_size, window, chunk, sink, scale, waves, shared, stream);
+}
+
+// The same with capped scores: softcap > 0, a scaled score s enters the softmax as softcap * tanh(s / softcap).
+extern "C" int tlie_attention_mfma_capped(const void* q, const void* cache, const int* block_table, int max_blocks,
+                                          const void* tiles, int num_tiles, int col_tiles, const int* positions, void* out,
+                                          float* part_o, float* part_ml, int nsplit, int split_len, int tokens, int nq, int nkv,
+                                          int d, int page_size, int window, int chunk, const float* sink, float scale, int waves,
+                                          int shared, float softcap, void* stream) {
+  return attention_entry(q, cache, block_table, max_blocks, tiles, num_tiles, col_tiles, positions, out, part_o, part_ml, nsplit,
+                         split_len, tokens, nq, nkv, d, page_size, window, chunk, sink, scale, waves, shared, stream, 0, softcap);
 }
 
 // The same with planes of a page that several kv heads share (see the kernel's plane_map): key_share kv heads in a row

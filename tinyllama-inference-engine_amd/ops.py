@@ -1685,7 +1685,8 @@ def attention_mfma(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tens
                    positions: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, window: int | None,
                    scale: float, nsplit: int = 1, split_len: int = 0, col_tiles: int = 1, waves: int = 1,
                    shared: bool = False, chunk: int | None = None, sink: torch.Tensor | None = None,
-                   planes: tuple[int, int, int] | None = None, float_out: bool = False) -> torch.Tensor:
+                   planes: tuple[int, int, int] | None = None, float_out: bool = False,
+                   softcap: float | None = None) -> torch.Tensor:
     """Causal attention of every token of the step over its sequence's cache, bfloat16.
 
     tiles: int32 [n, 4] from `attention_tiles` (built from the same step as block_table and
@@ -1705,8 +1706,11 @@ def attention_mfma(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tens
     a row the i-th reads value plane i % value_planes of that group's value_planes.  A page then holds
     nkv / key_share planes of keys and after them nkv / value_group * value_planes planes of values, each
     page_size * d (cache: [pages, ...] with so many values a page).  The result has all nq heads.
-    float_out (with planes): the result is float32."""
+    float_out (with planes): the result is float32.
+    softcap (without planes): a scaled score s enters the softmax as softcap * tanh(s / softcap)."""
     _device_tensor(q, "q", torch.bfloat16)
+    if softcap is not None and (not float(softcap) > 0.0 or planes is not None):
+        raise invalid_argument("attention: a cap of the scores must be positive, and does not go with shared planes")
     if planes is not None:
         key_share, value_group, value_planes = (int(v) for v in planes)
         if (min(key_share, value_group, value_planes) <= 0 or max(key_share, value_group) > 255 or value_planes > value_group
@@ -1777,6 +1781,14 @@ def attention_mfma(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tens
                                                     int(window) if window else 0, int(chunk) if chunk else 0, _ptr(sink),
                                                     ctypes.c_float(scale), waves, int(bool(shared)), key_share, value_group,
                                                     value_planes, 1 if float_out else 0, _stream()), "attention_mfma")
+        return out
+    if softcap is not None:
+        _check(library().tlie_attention_mfma_capped(_ptr(q), _ptr(cache), _ptr(block_table), block_table.shape[1], _ptr(tiles),
+                                                    num_tiles, col_tiles, _ptr(positions), _ptr(out), _ptr(part_o), _ptr(part_ml),
+                                                    nsplit, split_len, tokens, num_heads, num_kv_heads, head_dim, page_size,
+                                                    int(window) if window else 0, int(chunk) if chunk else 0, _ptr(sink),
+                                                    ctypes.c_float(scale), waves, int(bool(shared)), ctypes.c_float(softcap),
+                                                    _stream()), "attention_mfma")
         return out
     _check(library().tlie_attention_mfma(_ptr(q), _ptr(cache), _ptr(block_table), block_table.shape[1], _ptr(tiles),
                                          num_tiles, col_tiles, _ptr(positions), _ptr(out), _ptr(part_o), _ptr(part_ml), nsplit,

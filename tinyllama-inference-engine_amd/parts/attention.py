@@ -189,12 +189,12 @@ class Attention(Mixer):
                           rot_dim, binding.cache, self.nq, 0 if self.reads_other_cache else self.nkv, self.d, self.dv, self.dtype,
                           q_norm=self.q_norm, k_norm=self.k_norm, norm_eps=self.norm_eps, values_are_keys=self.values_are_keys,
                           q_temp=self.q_temp)
-        if self.dv == self.d and self.softcap is None and ops.attention_mfma_takes(self.dtype, self.d, binding.cache.shape[3] // self.d):
+        if self.dv == self.d and ops.attention_mfma_takes(self.dtype, self.d, binding.cache.shape[3] // self.d):
             # bfloat16, one head size: the kernel on the matrix cores (scores, softmax and sink float)
             tiles, col_tiles, nsplit, split_len, waves, shared = ops.attention_plan(ctx, self.nq // self.nkv, self.nkv, self.d)
             attended = ops.attention_mfma(q, binding.cache, pages.block_table, tiles, ctx.positions, self.nq, self.nkv, self.d,
                                           self.window, self.scale, nsplit, split_len, col_tiles, waves, shared,
-                                          chunk=self.chunk, sink=self.sink)
+                                          chunk=self.chunk, sink=self.sink, softcap=self.softcap)
         else:
             attended = ops.attention_generic(q, binding.cache, pages.block_table, ctx.token_seq, ctx.positions, self.nq, self.nkv,
                                              self.d, self.window, self.scale, tiled=ops.attention_generic_plan(ctx, self.d, self.dv),

@@ -90,7 +90,7 @@ class RoutedMLP(FeedForward):
         hidden = int(spec["hidden_size"])
         specs = [TensorSpec(prefix + names["router"], (int(spec["experts"]), hidden))]
         if spec.get("router_bias", False):
-            specs.append(TensorSpec(prefix + names["router_bias"], (int(spec["experts"]),), init="offset"))
+            specs.append(TensorSpec(prefix + names["router_bias"], (int(spec["experts"]),), init="spread"))
         if spec.get("shared_gate", False):
             specs.append(TensorSpec(prefix + names["shared_gate"], (1, hidden)))
         for place, size in cls._prefixes(spec, prefix, names):

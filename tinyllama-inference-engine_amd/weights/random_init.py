@@ -53,6 +53,9 @@ def _draw(spec: TensorSpec, seed: int, std: float, norm_std: float, dtype: torch
         # the weights of a sum of which the last summand is the main one
         values = values * 0.2
         values[..., -1] += 1.0
+    elif spec.init == "spread":
+        # numbers of order 1 whatever the other tensors' scale (a router's biases: they set the experts well apart)
+        values = values * 2.0
     elif spec.init == "near_identity":
         values = values * 0.15 + torch.eye(spec.shape[-1], device=device)
     elif spec.init == "share":
