@@ -265,12 +265,46 @@ def tugalix_configs(sizes):
     return tugalix, llama
 
 
+# layer sizes for `--design narolorn`: the same widths and vocabulary; attention layers with Llama's heads; a latent vector of 128
+# or 256 dims under as many heads; a routed feed-forward whose experts in use plus the shared one are as wide as the dense
+# feed-forward; four streams of the residual; four layers of which the first two run twice (six runs)
+NAROLORN_SIZES = {
+    "w2048": dict(width=2048, ff=5632, vocab=32000, streams=4, heads=32, kv_heads=4, dim=64, softcap=50.0, chunk=1024, window=1024,
+                  latent_heads=32, latent_dim=64, latent_vdim=64, rank=128, experts=8, top=2, expert_ff=1408, shared_ff=2816),
+    "w4096": dict(width=4096, ff=14336, vocab=32000, streams=4, heads=32, kv_heads=8, dim=128, softcap=50.0, chunk=1024, window=1024,
+                  latent_heads=32, latent_dim=128, latent_vdim=128, rank=256, experts=8, top=2, expert_ff=3584, shared_ff=7168),
+}
+
+
+def narolorn_configs(sizes):
+    """(the Narolorn configuration, the Llama configuration of equal sizes): windowed latent attention, chunked attention
+    whose values are its keys, attention with capped scores and a query temperature, latent attention again, each with a
+    routed feed-forward; the first two run twice.  Beside as many Llama layers as that makes runs."""
+    s = sizes
+    routed = {"kind": "moe", "expert": {"ff": s["expert_ff"], "limit": 7.0}, "router": {"experts": s["experts"], "top": s["top"]},
+              "shared": {"ff": s["shared_ff"], "limit": 7.0}}
+    scale = s["dim"] ** -0.5
+    latent = {"heads": s["latent_heads"], "dim": s["latent_dim"], "vdim": s["latent_vdim"], "kv_rank": s["rank"],
+              "scale": s["latent_dim"] ** -0.5, "mask": {"size": s["window"]}}
+    chunked = {"heads": s["heads"], "kv_heads": s["kv_heads"], "dim": s["dim"], "vdim": s["dim"], "scale": scale,
+               "mask": {"size": s["chunk"]}, "rot": {"base": 10000.0, "dims": s["dim"]}}
+    capped = {"heads": s["heads"], "kv_heads": s["kv_heads"], "dim": s["dim"], "vdim": s["dim"], "scale": scale, "softcap": s["softcap"],
+              "q_temp": {"coef": 0.1, "every": 512}}
+    layers = [{"type": "latent_attention", "mixer": latent, "mlp": routed}, {"type": "attention_2", "mixer": chunked, "mlp": routed},
+              {"type": "attention", "mixer": capped, "mlp": routed}, {"type": "latent_attention", "mixer": latent, "mlp": routed}]
+    narolorn = {"architecture": "Narolorn", "vocab": s["vocab"], "width": s["width"], "norm": {"eps": 1e-5}, "streams": s["streams"],
+                "logit_softcap": 30.0, "loop": {"start": 0, "stop": 2, "times": 2}, "layers": layers}
+    llama = dict(TINYLLAMA, hidden_size=s["width"], intermediate_size=s["ff"], num_hidden_layers=6,
+                 num_attention_heads=s["heads"], num_key_value_heads=s["kv_heads"], vocab_size=s["vocab"], max_position_embeddings=4096)
+    return narolorn, llama
+
+
 def bench_design(args, torch) -> int:
-    """`--design fadutar|raketar|tugalix`: one JSON line.  Per size: tokens a second of a prompt step of 2048 tokens and of decode steps
+    """`--design fadutar|raketar|tugalix|narolorn`: one JSON line.  Per size: tokens a second of a prompt step of 2048 tokens and of decode steps
     at the record's batch and context, for that decoder and for the Llama decoder of equal sizes (random
     weights, bfloat16, through the engine's own loop), and every kernel the design adds alone, beside the like kernel."""
     from tlie_amd import Engine, ops
-    from tlie_amd.kernel_bench import bench_design_kernels, bench_raketar_kernels, bench_tugalix_kernels
+    from tlie_amd.kernel_bench import bench_design_kernels, bench_narolorn_kernels, bench_raketar_kernels, bench_tugalix_kernels
     peaks = ops.measured_peaks("cuda:0")
     record = {"metric": f"{args.design}: prefill and decode tok/s beside the Llama decoder of equal sizes", "unit": "tokens/s",
               "n_gpus": 1, "dtype": "bf16", "data": "synthetic: uniform random token ids, random weights",
@@ -278,9 +312,10 @@ def bench_design(args, torch) -> int:
     steps, warmup = min(args.steps, 48), 4
     all_sizes, configs, kernels = {"fadutar": (DESIGN_SIZES, design_configs, bench_design_kernels),
                                    "raketar": (RAKETAR_SIZES, raketar_configs, bench_raketar_kernels),
-                                   "tugalix": (TUGALIX_SIZES, tugalix_configs, bench_tugalix_kernels)}[args.design]
+                                   "tugalix": (TUGALIX_SIZES, tugalix_configs, bench_tugalix_kernels),
+                                   "narolorn": (NAROLORN_SIZES, narolorn_configs, bench_narolorn_kernels)}[args.design]
     for name, sizes in all_sizes.items():
-        entry = {"layers": {"fadutar": 4 * sizes.get("groups", 0), "raketar": 6, "tugalix": 4}[args.design], "sizes": sizes}
+        entry = {"layers": {"fadutar": 4 * sizes.get("groups", 0), "raketar": 6, "tugalix": 4, "narolorn": 6}[args.design], "sizes": sizes}
         for model, config in zip((args.design, "llama"), configs(sizes)):
             engine = Engine(None, dtype="bfloat16", config=config, random_seed=0, max_tokens=args.batch * args.context + 4096,
                             page_size=16, max_requests=args.batch + 1)
@@ -326,7 +361,7 @@ def main() -> int:
                         help="time the kernels of a decode step (--batch, --context) and of a prompt step one by one at the "
                              "shape's layer sizes, each inside a replayed recording that walks through copies of its weights; "
                              "NAME keeps the kernels whose name holds it; prints one JSON line per kernel")
-    parser.add_argument("--design", default=None, choices=["fadutar", "raketar", "tugalix"],
+    parser.add_argument("--design", default=None, choices=["fadutar", "raketar", "tugalix", "narolorn"],
                         help="prefill and decode throughput of that decoder design at layer sizes of real models, beside the Llama "
                              "decoder at equal sizes, and its own kernels alone beside the like kernels (one JSON line of its own)")
     parser.add_argument("--shape", default="tinyllama", choices=["tinyllama", *OTHER_SHAPES],

@@ -486,6 +486,134 @@ def bench_raketar_kernels(sizes: dict, batch: int = 8, context: int = 2048, prom
     return rows
 
 
+
+def bench_narolorn_kernels(sizes: dict, batch: int = 8, context: int = 2048, prompt: int = 2048, samples: int = 10, device="cuda:0",
+                           hbm_gbs: float = 8000.0, mfma_tflops: float = 2500.0) -> list[dict]:
+    """The kernels that the Narolorn decoder adds or extends, each alone at a layer's sizes, for a decode step of `batch`
+    requests at `context` positions and a prompt step of `prompt` tokens, each beside the like kernel of the Llama decoder at
+    the same sizes; every row carries the fraction of the roofline its bytes or flops reach (`frac`: of `hbm_gbs` for rows
+    with bytes, of `mfma_tflops` for rows with flops).
+    sizes: width, ff, vocab, streams, heads, kv_heads, dim; softcap, chunk, window; latent_heads, latent_dim, latent_vdim, rank;
+    experts, top, expert_ff, shared_ff."""
+    device = torch.device(device)
+    torch.cuda.set_device(device)
+    bf, f32 = torch.bfloat16, torch.float32
+    width, ff, vocab, count = sizes["width"], sizes["ff"], sizes["vocab"], sizes["streams"]
+    H, G, d = sizes["heads"], sizes["kv_heads"], sizes["dim"]
+    lh, ld, lv, rank = sizes["latent_heads"], sizes["latent_dim"], sizes["latent_vdim"], sizes["rank"]
+    experts, top, eff, sff = sizes["experts"], sizes["top"], sizes["expert_ff"], sizes["shared_ff"]
+    page_size, rows = 16, []
+    units = int(torch.cuda.get_device_properties(device).multi_processor_count)
+
+    def rand(*shape, scale=0.02, dtype=bf):
+        return (torch.randn(shape, device=device, dtype=f32) * scale).to(dtype)
+
+    def row(name, times, read_bytes=0, flops=0):
+        entry = _row(name, times, read_bytes, flops)
+        if read_bytes:
+            entry["frac"] = round(entry["gbs"] / hbm_gbs, 3)
+        elif flops:
+            entry["frac"] = round(entry["tflops"] / mfma_tflops, 4)
+        rows.append(entry)
+
+    def ints(values):
+        return torch.tensor(values, dtype=torch.int32, device=device)
+
+    for label, tokens, seqs in ((f"decode b{batch}", batch, batch), (f"prompt {prompt}", prompt, 1)):
+        if tokens <= 0:
+            continue
+        decode = seqs == tokens
+        length = context if decode else prompt
+        blocks = (length + page_size - 1) // page_size
+        table = torch.arange(seqs * blocks, dtype=torch.int32, device=device).view(seqs, blocks).contiguous()
+        if decode:
+            positions = torch.full((tokens,), length - 1, dtype=torch.int32, device=device)
+            token_seq = ints(list(range(tokens)))
+            host = {"seq_start": np.arange(tokens + 1, dtype=np.int32), "seq_len": np.full(tokens, length, dtype=np.int32)}
+        else:
+            positions = torch.arange(tokens, dtype=torch.int32, device=device)
+            token_seq = torch.zeros(tokens, dtype=torch.int32, device=device)
+            host = {"seq_start": np.asarray([0, tokens], dtype=np.int32), "seq_len": np.asarray([tokens], dtype=np.int32)}
+        slot_map = (table[token_seq.long(), (positions // page_size).long()] * page_size + positions % page_size).to(torch.int32).contiguous()
+        ctx = SimpleNamespace(max_new=1 if decode else tokens, num_seqs=seqs, num_tokens=tokens, max_context=length, scratch={},
+                              tile_owner=None, compute_units=units, host=host, tokens=positions)
+        keys_seen = length if decode else (length + 1) / 2            # keys a token sees on average
+        # ---- attention: capped scores; chunks; the window over the latent cache; beside the plain causal one --------
+        cache = rand(seqs * blocks, 2, G, page_size * d, scale=0.5)
+        q = rand(tokens, H * d, scale=1.0)
+        cache_bytes, flops = seqs * length * G * 2 * d * 2, 4.0 * tokens * H * d * keys_seen
+        for name, options in (("causal (Llama's)", {}), ("capped scores", {"softcap": sizes["softcap"]}), (f"chunks of {sizes['chunk']}", {"chunk": sizes["chunk"]})):
+            ctx.scratch = {}
+            tiles, col_tiles, nsplit, split_len, waves, shared = ops.attention_plan(ctx, H // G, G, d)
+            times = _timed(lambda i: ops.attention_mfma(q, cache, table, tiles, positions, H, G, d, None, d ** -0.5, nsplit, split_len,
+                                                        col_tiles, waves, shared, **options), 8, samples)
+            seen = min(keys_seen, sizes["chunk"] if decode else sizes["chunk"] / 2) if "chunk" in options else keys_seen
+            row(f"{label}: attention, {name}, {H} heads of {d} on {G}", times, int(cache_bytes * seen / keys_seen) if decode else 0,
+                0 if decode else 4.0 * tokens * H * d * seen)
+        key = rank
+        latent_cache = rand(seqs * blocks, 2, 1, page_size * key, scale=0.5)
+        q_wide = rand(tokens, lh * key, scale=1.0)
+        ctx.scratch = {}
+        tiles, col_tiles, nsplit, split_len, waves, shared = ops.attention_plan(ctx, lh, 1, key)
+        times = _timed(lambda i: ops.attention_mfma(q_wide, latent_cache, table, tiles, positions, lh, 1, key, sizes["window"], ld ** -0.5,
+                                                    nsplit, split_len, col_tiles, waves, shared), 8, samples)
+        seen = min(keys_seen, sizes["window"])
+        row(f"{label}: attention over the latent cache, window of {sizes['window']}, {lh} heads on one key of {key}", times,
+            int(seqs * seen * 2 * key * 2) if decode else 0, 0 if decode else 4.0 * tokens * lh * key * seen)
+        # ---- placement ---------------------------------------------------------------------------------------------------
+        inv_freq = torch.ones(d // 2, device=device)
+        qkv = ops.Product(rand(tokens, (H + 2 * G) * d, scale=1.0), 1)
+        times = _timed(lambda i: ops.rope_cache(qkv, positions, slot_map, inv_freq, d, cache, H, G, d, bf), 8, samples)
+        row(f"{label}: rotation + cache write (Llama's)", times, tokens * (H * 2 + 2 * G) * d * 2 * 2)
+        times = _timed(lambda i: ops.qkv_place(qkv, positions, slot_map, None, 0, cache, H, G, d, d, bf, q_temp=(0.1, 512.0)), 8, samples)
+        row(f"{label}: placement of q, k, v with a query temperature", times, tokens * (H * 2 + 2 * G) * d * 2 * 2)
+        qk = ops.Product(rand(tokens, (H + G) * d, scale=1.0), 1)
+        q_norm, k_norm = rand(H * d, scale=1.0, dtype=f32), rand(G * d, scale=1.0, dtype=f32)
+        times = _timed(lambda i: ops.qkv_place(qk, positions, slot_map, inv_freq, d, cache, H, G, d, d, bf, q_norm=q_norm, k_norm=k_norm,
+                                               norm_eps=1e-5, values_are_keys=True), 8, samples)
+        row(f"{label}: placement of q and k: norms over the whole projections, rotation, the projected keys as values", times,
+            tokens * ((H + G) * d * 2 * 2 + G * d * 2))
+        gate_cols = lh * lv
+        fused = ops.Product(rand(tokens, lh * ld + rank + gate_cols, scale=1.0), 1)
+        latent_norm = rand(rank, scale=1.0)
+        times = _timed(lambda i: ops.latent_place(fused, positions, slot_map, None, latent_norm, 1e-5, latent_cache, lh, ld, 0, rank, bf,
+                                                  wide_values=True, turn=0, extra_cols=gate_cols), 8, samples)
+        row(f"{label}: latent placement (norm, cache write, queries apart)", times, tokens * (lh * ld * 2 + rank * 3) * 2)
+        values = rand(tokens, gate_cols, scale=1.0)
+        times = _timed(lambda i: ops.sigmoid_gate(values, fused, fused.cols - gate_cols), 8, samples)
+        row(f"{label}: gate on the heads' results", times, tokens * gate_cols * 6)
+        # ---- the residual of several streams ------------------------------------------------------------------------------
+        streams = rand(count, tokens, width, scale=1.0, dtype=f32)
+        update = ops.StreamUpdate(ops.Product(rand(tokens, width, scale=1.0), 1), rand(count, count, scale=0.3, dtype=f32),
+                                  rand(count, scale=0.3, dtype=f32))
+        read, norm_w = rand(count, scale=0.5, dtype=f32), rand(width, scale=1.0)
+        times = _timed(lambda i: ops.stream_norm(streams, update, read, norm_w, 1e-5, bf), 8, samples)
+        row(f"{label}: {count} streams take a result, are read and normed", times, tokens * width * (count * 8 + 2 + 2))
+        times = _timed(lambda i: ops.stream_norm(streams, update, None, None, 0.0, bf, total=True), 8, samples)
+        row(f"{label}: {count} streams take a result and are summed", times, tokens * width * (count * 8 + 2 + 4))
+        residual = rand(tokens, width, scale=1.0, dtype=f32)
+        times = _timed(lambda i: ops.add_rmsnorm(residual, update.product, norm_w, 1e-5, bf), 8, samples)
+        row(f"{label}: add + norm (Llama's)", times, tokens * width * (4 + 4 + 2 + 2))
+        # ---- the routed feed-forward --------------------------------------------------------------------------------------
+        x = rand(tokens, width, scale=1.0)
+        router, bias = rand(experts + 1, width), rand(experts + 1)
+        times = _timed(lambda i: ops.few_outputs(x, router, bias, top=top, score="softmax_of_chosen", extra=1), 8, samples)
+        row(f"{label}: router, softmax over the chosen {top} of {experts}, the shared expert's gate", times, (tokens + experts + 1) * width * 2)
+        inter = experts * eff + sff
+        scale = ops.few_outputs(x, router, bias, top=top, score="softmax_of_chosen", extra=1)
+        gate_up = ops.Product(rand(tokens, 2 * inter, scale=1.0), 1)
+        times = _timed(lambda i: ops.routed_gate(gate_up, scale, eff, bf, weigh="output", shared_scaled=True, gate="clamped_swish",
+                                                 alpha=1.702, limit=7.0, shared_limit=7.0), 4, samples)
+        row(f"{label}: clamped gate of the routed feed-forward, weighed results (all experts' columns)", times, tokens * inter * 6)
+        dense_up = ops.Product(rand(tokens, 2 * ff, scale=1.0), 1)
+        times = _timed(lambda i: ops.silu_mul(dense_up, bf, interleaved=True), 4, samples)
+        row(f"{label}: SiLU gate (Llama's)", times, tokens * ff * 6)
+        # ---- capped logits (the wanted rows: every row of a decode step, one of a prompt) ------------------------------
+        logits = rand(tokens if decode else 1, vocab, scale=5.0, dtype=f32)
+        times = _timed(lambda i: ops.softcap(logits, 30.0), 8, samples)
+        row(f"{label}: capped logits", times, logits.numel() * 8)
+    return rows
+
 def bench_tugalix_kernels(sizes: dict, batch: int = 8, context: int = 2048, prompt: int = 2048, samples: int = 10, device="cuda:0",
                           hbm_gbs: float = 8000.0, mfma_tflops: float = 2500.0) -> list[dict]:
     """The kernels that the Tugalix decoder adds, each alone at a layer's sizes, for a decode step of `batch` requests at
