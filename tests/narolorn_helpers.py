@@ -78,8 +78,8 @@ CONFIG_R = {        # one stream (the three small tensors still act), a loop of 
         {"type": "latent_attention", "mixer": _latent(4, 32, 32, 64, 0.18, window=24), "mlp": _moe(6, 2, 16, 3.0, (64, 1.0))},
     ],
 }
-CONFIG_S = {        # four streams, no loop
-    "architecture": "Narolorn", "vocab": 70, "width": 48, "norm": {"eps": 1e-5}, "streams": 4,
+CONFIG_S = {        # four streams, no loop; a width that is no multiple of four
+    "architecture": "Narolorn", "vocab": 70, "width": 50, "norm": {"eps": 1e-5}, "streams": 4,
     "layers": [
         {"type": "latent_attention", "mixer": _latent(2, 12, 12, 24, 0.3, window=3), "mlp": _moe(2, 2, 8, 2.0)},
         {"type": "attention", "mixer": _attention(2, 2, 8, 8, 0.4, q_temp=(1.0, 2)), "mlp": None},

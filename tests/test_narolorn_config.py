@@ -57,6 +57,9 @@ def test_the_expected_tensors_carry_the_designs_names_and_shapes():
     assert shapes["l1.mix.uv"] == (60, 48) and shapes["l1.mix.g"] == (60, 80) and "l1.mlp.shared.gate" not in shapes
     assert shapes["l2.mix.q.norm"] == (128,) and shapes["l2.mix.k.norm"] == (64,) and "l2.mix.v" not in shapes
     assert "l2.hc2.in" not in shapes and "l2.norm2" not in shapes          # a layer without a feed-forward
+    import re
+    assert any(re.fullmatch(pattern, "l2.norm2") for pattern in spec_of(CONFIG_P).ignored_tensors)      # (a file may still carry them)
+    assert not any(re.fullmatch(pattern, "l1.norm2") for pattern in spec_of(CONFIG_P).ignored_tensors)
     single = {tensor.name for tensor in expected_tensors(spec_of(CONFIG_Q))}
     assert not any(".hc" in name for name in single)
 

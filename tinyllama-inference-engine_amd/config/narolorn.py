@@ -151,6 +151,9 @@ class NarolornConfig:
                 mixer_norm_place="norm1", mixer_place="mix.", feed_forward_norm_place="norm2", feed_forward_place="mlp.",
                 streams=streams, mixer_streams_place="hc1.", feed_forward_streams_place="hc2."))
         count = len(layers)
+        # a layer without a feed-forward reads neither a second norm nor the second sublayer's stream tensors: a file that
+        # carries them all the same is taken, and they are left unread
+        ignored = tuple(rf"l{index}\.(norm2|hc2\.(in|out|mix))" for index, layer in enumerate(raw["layers"]) if layer.get("mlp") is None)
         order = list(range(count))
         loop = raw.get("loop")
         if loop is not None:
@@ -165,7 +168,8 @@ class NarolornConfig:
             architecture=self.architecture, hidden_size=width, vocab_size=vocab, max_positions=None,
             embedding=PartSpec("token_embedding", {"vocab_size": vocab, "hidden_size": width}),
             layers=tuple(layers), runs=tuple(runs), final_norm=norm, head=PartSpec("lm_head", head),
-            embedding_name="embed", final_norm_prefix="final.norm", head_name="head", streams=streams)
+            embedding_name="embed", final_norm_prefix="final.norm", head_name="head", streams=streams,
+            ignored_tensors=ignored)
         spec.validate()
         return spec
 

@@ -269,6 +269,23 @@ __global__ void sigmoid_gate_kernel(A* __restrict__ values, const D* __restrict_
   }
 }
 
+// The same with eight columns a thread (no partial sums, cols, col and row_width multiples of 8, 16-byte aligned arrays).
+template <typename D, typename A>
+__global__ void sigmoid_gate_wide_kernel(A* __restrict__ values, const D* __restrict__ pre, int col, int row_width, size_t groups, int cols) {
+  const int per_row = cols / 8;
+  for (size_t index = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; index < groups;
+       index += static_cast<size_t>(gridDim.x) * blockDim.x) {
+    const size_t t = index / per_row;
+    const int c = static_cast<int>(index % per_row) * 8;
+    float v[8], z[8];
+    load8(values + t * cols + c, v);
+    load8(pre + t * row_width + col + c, z);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = v[j] / (1.f + expf(-z[j]));
+    store8(values + t * cols + c, v);
+  }
+}
+
 // ---- x <- cap * tanh(x / cap), in place (capped logits) --------------------------------------------------------------
 __global__ void softcap_kernel(float* __restrict__ x, size_t total, float cap) {
   for (size_t index = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; index < total;
@@ -445,8 +462,20 @@ extern "C" int tlie_sigmoid_gate(void* values, int act_dtype, const void* pre, i
                                  int col, int row_width, int rows, int cols, void* stream) {
   if (rows <= 0 || cols <= 0 || col < 0 || col + cols > row_width || nsplit < 1) return kBadArgument;
   const size_t total = static_cast<size_t>(rows) * cols;
-  const int blocks = static_cast<int>((total + 255) / 256 < 16384 ? (total + 255) / 256 : 16384);
   hipStream_t s = (hipStream_t)stream;
+  if (nsplit == 1 && cols % 8 == 0 && col % 8 == 0 && row_width % 8 == 0 && pre_dtype == act_dtype &&
+      ((reinterpret_cast<uintptr_t>(values) | reinterpret_cast<uintptr_t>(pre)) & 31) == 0) {
+    const size_t groups = total / 8;
+    const int wide_blocks = static_cast<int>((groups + 255) / 256 < 16384 ? (groups + 255) / 256 : 16384);
+    if (act_dtype == kBF16)
+      hipLaunchKernelGGL((sigmoid_gate_wide_kernel<bf16, bf16>), dim3(wide_blocks), dim3(256), 0, s, (bf16*)values, (const bf16*)pre, col,
+                         row_width, groups, cols);
+    else
+      hipLaunchKernelGGL((sigmoid_gate_wide_kernel<float, float>), dim3(wide_blocks), dim3(256), 0, s, (float*)values, (const float*)pre,
+                         col, row_width, groups, cols);
+    return launch_status();
+  }
+  const int blocks = static_cast<int>((total + 255) / 256 < 16384 ? (total + 255) / 256 : 16384);
 #define TLIE_CASE(DC, D, AC, A)                                                                                  \
   if (pre_dtype == DC && act_dtype == AC) {                                                                      \
     hipLaunchKernelGGL((sigmoid_gate_kernel<D, A>), dim3(blocks), dim3(256), 0, s, (A*)values, (const D*)pre, nsplit, \

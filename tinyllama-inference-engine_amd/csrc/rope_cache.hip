@@ -157,6 +157,7 @@ struct PlaceOptions {
   int values_are_keys;
   float temp_coef;
   float temp_every;
+  int stage;         // the launch gave LDS for the q and k columns (set by the entry point)
 };
 
 template <typename D, typename A>
@@ -170,36 +171,36 @@ __global__ void qkv_place_kernel(const D* __restrict__ qkv, int nsplit, size_t s
   float* cosines = lds;                  // half
   float* sines = cosines + half;         // half
   float* scratch = sines + half;         // 16
+  float* staged = scratch + 16;          // the q and k columns as floats, when the launch gave the room (stage != 0)
   const int t = blockIdx.x;
   const int rotated = (nq + nkv) * d, width = rotated + (options.values_are_keys ? 0 : nv * dv);
   const D* in = qkv + static_cast<size_t>(t) * row_width;
   if (inv_freq != nullptr) {
     const float pos = static_cast<float>(positions[t]);
     for (int i = threadIdx.x; i < half; i += blockDim.x) sincosf(pos * inv_freq[i], &sines[i], &cosines[i]);
-    __syncthreads();
   }
+  // With norms every q and k column is needed three times (its projection's sum of squares, itself, its rotation
+  // partner): they are read once, into LDS, and the sums of squares are formed on the way.
+  const bool stage = options.stage != 0;
+  auto raw = [&](int c) { return stage ? staged[c] : sum_splits(in + c, nsplit, split_stride); };
   float q_scale = 1.f, k_scale = 1.f;
-  if (options.q_norm != nullptr) {
-    float square = 0.f;
-    for (int c = threadIdx.x; c < nq * d; c += blockDim.x) {
+  if (options.q_norm != nullptr || options.k_norm != nullptr) {
+    float q_square = 0.f, k_square = 0.f;
+    for (int c = threadIdx.x; c < rotated; c += blockDim.x) {
       const float v = sum_splits(in + c, nsplit, split_stride);
-      square += v * v;
+      if (stage) staged[c] = v;
+      if (c < nq * d) q_square += v * v;
+      else k_square += v * v;
     }
-    q_scale = rsqrtf(block_sum(square, scratch) / static_cast<float>(nq * d) + options.eps);
+    if (options.q_norm != nullptr) q_scale = rsqrtf(block_sum(q_square, scratch) / static_cast<float>(nq * d) + options.eps);
+    if (options.k_norm != nullptr && nkv > 0) k_scale = rsqrtf(block_sum(k_square, scratch) / static_cast<float>(nkv * d) + options.eps);
   }
-  if (options.k_norm != nullptr && nkv > 0) {
-    float square = 0.f;
-    for (int c = nq * d + threadIdx.x; c < rotated; c += blockDim.x) {
-      const float v = sum_splits(in + c, nsplit, split_stride);
-      square += v * v;
-    }
-    k_scale = rsqrtf(block_sum(square, scratch) / static_cast<float>(nkv * d) + options.eps);
-  }
+  __syncthreads();                       // the angles and the staged columns are written
   if (options.temp_every > 0.f)
     q_scale *= 1.f + options.temp_coef * logf(floorf(static_cast<float>(positions[t] + 1) / options.temp_every) + 1.f);
   // a column of q or k after its norm (and, for a query, its temperature), before the rotation
   auto normed = [&](int c) {
-    const float v = sum_splits(in + c, nsplit, split_stride);
+    const float v = raw(c);
     if (c < nq * d) return options.q_norm != nullptr ? v * q_scale * options.q_norm[c] : v * q_scale;
     return options.k_norm != nullptr ? v * k_scale * options.k_norm[c - nq * d] : v;
   };
@@ -225,8 +226,7 @@ __global__ void qkv_place_kernel(const D* __restrict__ qkv, int nsplit, size_t s
     } else {
       page[(static_cast<size_t>(head - nq) * page_size + row) * d + e] = from_float<A>(v);
       if (options.values_are_keys)
-        page[static_cast<size_t>(nkv) * page_size * d + (static_cast<size_t>(head - nq) * d + e) * page_size + row] =
-            from_float<A>(sum_splits(in + c, nsplit, split_stride));
+        page[static_cast<size_t>(nkv) * page_size * d + (static_cast<size_t>(head - nq) * d + e) * page_size + row] = from_float<A>(raw(c));
     }
   }
 }
@@ -252,9 +252,15 @@ extern "C" int tlie_qkv_place(const void* qkv, int in_dtype, int nsplit, long lo
   if (temp_every < 0.f) return kBadArgument;
   const int width = (nq + nkv) * d + (values_are_keys ? 0 : nv * dv);
   if (row_width < width) return kBadArgument;
-  const int threads = width >= 1024 ? 1024 : (width + 63) / 64 * 64;
-  const size_t lds = (static_cast<size_t>(rot_dim) + 16) * sizeof(float);
-  const PlaceOptions options{q_norm, k_norm, norm_eps, values_are_keys, temp_coef, temp_every};
+  int threads = width >= 1024 ? 1024 : (width + 63) / 64 * 64;
+  // with norms a workgroup waits several times for all its waves (two sums over the row); in a step of many tokens
+  // smaller workgroups, more of which fit a compute unit, fill those waits with each other's work
+  if ((q_norm != nullptr || k_norm != nullptr) && tokens > 64 && threads > 256) threads = 256;
+  const bool normed = q_norm != nullptr || k_norm != nullptr;
+  const size_t columns = static_cast<size_t>(nq + nkv) * d;
+  const int stage = normed && columns <= 14000 ? 1 : 0;          // (beyond that a row does not fit beside the rest: every read goes to memory)
+  const size_t lds = (static_cast<size_t>(rot_dim) + 16 + (stage ? columns : 0)) * sizeof(float);
+  const PlaceOptions options{q_norm, k_norm, norm_eps, values_are_keys, temp_coef, temp_every, stage};
   hipStream_t s = (hipStream_t)stream;
 #define TLIE_CASE(DC, D, AC, A)                                                                                \
   if (in_dtype == DC && act_dtype == AC) {                                                                     \

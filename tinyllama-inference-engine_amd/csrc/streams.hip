@@ -13,15 +13,15 @@
 //   total != null    the sum of the (updated) streams is written there, [tokens][hidden] floats: what the
 //                    model's last norm reads
 // A token is a workgroup's; a thread holds the S values of a column in registers, so the update in place
-// reads every old value before it writes a new one.  Everything is float.  S <= kMaxStreams.
+// reads every old value before it writes a new one.  Everything is float.  S <= kStreamsLimit.
 #include "common.h"
 
 namespace tlie {
 
-constexpr int kMaxStreams = 8;
+constexpr int kStreamsLimit = 8;     // the kernel is built for up to 4 streams (up to 1024 threads a token) and for up to 8
 
-template <typename D, typename W, typename O, int VEC>
-__global__ void __launch_bounds__(256)
+template <typename D, typename W, typename O, int VEC, int kMaxStreams>
+__global__ void __launch_bounds__(kMaxStreams <= 4 ? 1024 : 256)
 stream_norm_kernel(float* __restrict__ streams, size_t stream_stride, int count, const D* __restrict__ delta, int nsplit,
                    size_t split_stride, const float* __restrict__ mix, const float* __restrict__ write,
                    const float* __restrict__ read, const W* __restrict__ weight, float eps, O* __restrict__ out,
@@ -53,8 +53,19 @@ stream_norm_kernel(float* __restrict__ streams, size_t stream_stride, int count,
       }
     }
     if (delta != nullptr) {
+      const D* part = delta + static_cast<size_t>(t) * hidden + i;
+      if constexpr (VEC == 4 && sizeof(D) == 4) {
+        // partial sums of a split product, four columns a load, added in the order of their index
+        float4 sum = *reinterpret_cast<const float4*>(part);
+        for (int split = 1; split < nsplit; ++split) {
+          const float4 more = *reinterpret_cast<const float4*>(part + split * split_stride);
+          sum.x += more.x; sum.y += more.y; sum.z += more.z; sum.w += more.w;
+        }
+        y[0] = sum.x; y[1] = sum.y; y[2] = sum.z; y[3] = sum.w;
+      } else {
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) y[j] = sum_splits(delta + static_cast<size_t>(t) * hidden + i + j, nsplit, split_stride);
+        for (int j = 0; j < VEC; ++j) y[j] = sum_splits(part + j, nsplit, split_stride);
+      }
       float fresh[kMaxStreams][VEC];
 #pragma unroll
       for (int r = 0; r < kMaxStreams; ++r) {
@@ -94,8 +105,9 @@ stream_norm_kernel(float* __restrict__ streams, size_t stream_stride, int count,
       square += u[j] * u[j];
     }
     if (read != nullptr) {
+      // (u times the norm's weight waits in LDS: the second pass then only applies the row's scale)
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) row_cache[i + j] = u[j];
+      for (int j = 0; j < VEC; ++j) row_cache[i + j] = u[j] * to_float(weight[i + j]);
     }
     if (total != nullptr) {
 #pragma unroll
@@ -107,7 +119,7 @@ stream_norm_kernel(float* __restrict__ streams, size_t stream_stride, int count,
   O* o = out + static_cast<size_t>(t) * hidden;
   for (int i = threadIdx.x * VEC; i < hidden; i += blockDim.x * VEC) {
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) o[i + j] = from_float<O>(row_cache[i + j] * scale * to_float(weight[i + j]));   // (the thread's own entries)
+    for (int j = 0; j < VEC; ++j) o[i + j] = from_float<O>(row_cache[i + j] * scale);   // (the thread's own entries)
   }
 }
 
@@ -130,27 +142,39 @@ using namespace tlie;
 extern "C" int tlie_stream_norm(float* streams, int count, const void* delta, int delta_dtype, int nsplit, long long split_stride,
                                 const float* mix, const float* write, const float* read, const void* weight, int weight_dtype,
                                 float eps, void* out, int out_dtype, float* total, int tokens, int hidden, void* stream) {
-  if (tokens <= 0 || hidden <= 0 || count <= 0 || count > kMaxStreams || nsplit < 1) return kBadArgument;
+  if (tokens <= 0 || hidden <= 0 || count <= 0 || count > kStreamsLimit || nsplit < 1) return kBadArgument;
   if (delta != nullptr && (mix == nullptr || write == nullptr)) return kBadArgument;
   if (read != nullptr && (weight == nullptr || out == nullptr || !(eps > 0.f))) return kBadArgument;
   const size_t lds = (static_cast<size_t>(read != nullptr ? hidden : 0) + 16) * sizeof(float);
   if (lds > 64 * 1024) return kBadArgument;
   const size_t stride = static_cast<size_t>(tokens) * hidden;
-  const bool wide = (hidden & 3) == 0 && ((reinterpret_cast<uintptr_t>(streams) | reinterpret_cast<uintptr_t>(total)) & 15) == 0;
+  const bool wide = (hidden & 3) == 0 && (split_stride & 3) == 0 &&
+                    ((reinterpret_cast<uintptr_t>(streams) | reinterpret_cast<uintptr_t>(total) | reinterpret_cast<uintptr_t>(delta)) & 15) == 0;
   const int per_thread = wide ? 4 : 1;
   const int wanted = (hidden / per_thread + 63) / 64 * 64;
-  const int threads = wanted > 256 ? 256 : wanted;
+  // a step of few tokens has few workgroups: each then takes as many threads as its row has pieces, so that every load
+  // of the row is asked for at once (up to 4 streams; beyond, the registers of 256 threads)
+  const int most = count <= 4 && tokens <= 64 ? 1024 : 256;
+  const int threads = wanted > most ? most : wanted;
   hipStream_t s = (hipStream_t)stream;
   if (delta == nullptr) delta_dtype = kF32;
   if (read == nullptr) weight_dtype = kF32, out_dtype = kF32;
 #define TLIE_CASE(DC, D, WC, W, OC, O)                                                                                  \
   if (delta_dtype == DC && weight_dtype == WC && out_dtype == OC) {                                                     \
-    if (wide)                                                                                                           \
-      hipLaunchKernelGGL((stream_norm_kernel<D, W, O, 4>), dim3(tokens), dim3(threads), lds, s, streams, stride, count,  \
+    if (wide && count <= 4)                                                                                             \
+      hipLaunchKernelGGL((stream_norm_kernel<D, W, O, 4, 4>), dim3(tokens), dim3(threads), lds, s, streams, stride, count, \
+                         (const D*)delta, nsplit, (size_t)split_stride, mix, write, read, (const W*)weight, eps, (O*)out, \
+                         total, hidden);                                                                                \
+    else if (wide)                                                                                                      \
+      hipLaunchKernelGGL((stream_norm_kernel<D, W, O, 4, 8>), dim3(tokens), dim3(threads), lds, s, streams, stride, count, \
+                         (const D*)delta, nsplit, (size_t)split_stride, mix, write, read, (const W*)weight, eps, (O*)out, \
+                         total, hidden);                                                                                \
+    else if (count <= 4)                                                                                                \
+      hipLaunchKernelGGL((stream_norm_kernel<D, W, O, 1, 4>), dim3(tokens), dim3(threads), lds, s, streams, stride, count, \
                          (const D*)delta, nsplit, (size_t)split_stride, mix, write, read, (const W*)weight, eps, (O*)out, \
                          total, hidden);                                                                                \
     else                                                                                                                \
-      hipLaunchKernelGGL((stream_norm_kernel<D, W, O, 1>), dim3(tokens), dim3(threads), lds, s, streams, stride, count,  \
+      hipLaunchKernelGGL((stream_norm_kernel<D, W, O, 1, 8>), dim3(tokens), dim3(threads), lds, s, streams, stride, count, \
                          (const D*)delta, nsplit, (size_t)split_stride, mix, write, read, (const W*)weight, eps, (O*)out, \
                          total, hidden);                                                                                \
     return launch_status();                                                                                             \
