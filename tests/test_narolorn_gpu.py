@@ -600,3 +600,22 @@ def test_drawn_configurations_in_bfloat16(tmp_path, seed):
     cut = run_cut(engine, "c", tokens, [50] + [1] * 20)
     assert_settled(cut, setup, tokens, "bfloat16", TOLERANCE["bfloat16"], f"seed {seed}, the last tokens one by one: {raw}", least=0.0)
     engine.cache.check()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_latent_vector_wider_than_any_value_head(tmp_path, dtype):
+    """A latent vector of 320 dims is beyond what the attention kernels take as a value head: the layer then expands and
+    caches every head's keys and values; the results are the same function of the weights."""
+    from tlie_amd import Engine
+    raw = {"architecture": "Narolorn", "vocab": 90, "width": 72, "norm": {"eps": 1e-5}, "streams": 2,
+           "layers": [{"type": "latent_attention", "mixer": {"heads": 3, "dim": 16, "vdim": 16, "kv_rank": 320, "scale": 0.25, "mask": {"size": 21}},
+                       "mlp": None},
+                      {"type": "latent_attention", "mixer": {"heads": 2, "dim": 8, "vdim": 24, "kv_rank": 272, "scale": 0.3}, "mlp": None}]}
+    folder = make_model(tmp_path / "model", raw, seed=5)
+    config, weights = load_plain(folder)
+    tokens = tokens_of(9, 60, raw["vocab"])
+    want = plain.forward(config, weights, tokens)[0]
+    engine = Engine(folder, dtype=dtype, max_tokens=128, page_size=16, max_requests=2)
+    for cuts in ([len(tokens)], [1], [7, 2, 30, 1]):
+        assert_rows(run_cut(engine, "r", tokens, cuts), want, TOLERANCE[dtype], f"{dtype} cut {cuts}")
+    engine.cache.check()

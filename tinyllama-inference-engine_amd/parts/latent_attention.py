@@ -66,9 +66,13 @@ class LatentAttention(Mixer):
             raise invalid_config("latent_attention: a window must be a positive count of positions")
         if min(self.heads, self.plain, self.dv, self.rank) <= 0 or self.rot < 0:
             raise invalid_config("latent_attention: sizes must be positive")
-        if self.rank > ops.ATTENTION_MAX_HEAD_DIM:
+        # A latent vector wider than the attention kernels' value heads cannot be attended over as it is: the layer then
+        # expands every position's keys and values once, when the position is placed, and caches those (per head, as an
+        # ordinary attention layer does); without a rotated part only.
+        self.expanded = self.rank > ops.ATTENTION_MAX_HEAD_DIM
+        if self.expanded and (self.rot > 0 or max(self.plain, self.dv) > ops.ATTENTION_MAX_HEAD_DIM):
             raise invalid_config(f"latent_attention: a latent vector of {self.rank} dims is beyond the attention kernel's "
-                                 f"{ops.ATTENTION_MAX_HEAD_DIM} value dims")
+                                 f"{ops.ATTENTION_MAX_HEAD_DIM} value dims, and the layer's heads cannot be expanded instead")
         # values as wide as keys while that is a head size the attention kernels take
         self.wide_values = self.rank + self.rot <= ops.ATTENTION_MAX_HEAD_DIM
         self.inv_freq, self.turn = None, 0             # turn: how many of the rot dims are rotated (the first ones)
@@ -118,21 +122,55 @@ class LatentAttention(Mixer):
             self.up_keys_rows = keep(self.up_keys.transpose(1, 2).contiguous())
             self.up_values_rows = keep(weights[prefix + names["up_values"]].reshape(self.heads, self.dv, self.rank).contiguous())
         self.o = Linear(weights[prefix + names["o"]], None, self.dtype, keep=keep)
+        self.expand = None
+        if self.expanded:
+            # one product from the normed latent vector to all heads' keys and values
+            self.expand = Linear(torch.cat([weights[prefix + names["up_keys"]], weights[prefix + names["up_values"]]], dim=0), None,
+                                 self.dtype, keep=keep)
         if self.has_sink:
             self.sink = keep(weights[prefix + names["sink"]].float().contiguous())
 
     def cache_need(self):
         """One key head of rank + rot dims, [row][dim], then its value dims transposed, [dim][row]: rank of them, or
         with wide values as many as a key has."""
+        if self.expanded:       # every head's keys and values, as an attention layer keeps them
+            if self.dv == self.plain:
+                return CacheNeed((2, self.heads), self.plain, self.window)
+            return CacheNeed((self.heads,), self.plain + self.dv, self.window)
         if self.wide_values:
             return CacheNeed((2, 1), self.rank + self.rot, self.window)
         return CacheNeed((1,), 2 * self.rank + self.rot, self.window)
+
+    def _forward_expanded(self, fused, ctx, binding: Binding):
+        """The latent vector is normed, every head's keys and values are formed from it by one product and placed in pages
+        of their own, and the attention runs over them head by head (window and sink as in the other form)."""
+        pages = ctx.groups[binding.group]
+        q_width = self.heads * self.plain
+        latent = fused.dense(torch.float32)[:, q_width:q_width + self.rank].contiguous()
+        c = ops.add_rmsnorm(latent, None, self.down_norm, self.norm_eps, self.dtype)
+        expanded = ops.as_product(self.expand(c)).dense(self.dtype)
+        qkv = ops.Product(torch.cat([fused.dense(self.dtype)[:, :q_width], expanded], dim=1).contiguous(), 1)
+        q = ops.qkv_place(qkv, ctx.positions, pages.slot_map if binding.writes else ctx.no_slots, None, 0, binding.cache, self.heads,
+                          self.heads, self.plain, self.dv, self.dtype)
+        if self.dv == self.plain and ops.attention_mfma_takes(self.dtype, self.plain, binding.cache.shape[3] // self.plain):
+            tiles, col_tiles, nsplit, split_len, waves, shared = ops.attention_plan(ctx, 1, self.heads, self.plain)
+            attended = ops.attention_mfma(q, binding.cache, pages.block_table, tiles, ctx.positions, self.heads, self.heads, self.plain,
+                                          self.window, self.scale, nsplit, split_len, col_tiles, waves, shared, sink=self.sink)
+        else:
+            attended = ops.attention_generic(q, binding.cache, pages.block_table, ctx.token_seq, ctx.positions, self.heads, self.heads,
+                                             self.plain, self.window, self.scale, tiled=ops.attention_generic_plan(ctx, self.plain, self.dv),
+                                             seq_start=ctx.seq_start, value_dim=self.dv, sink=self.sink)
+        if self.output_gate:
+            ops.sigmoid_gate(attended, fused, fused.cols - self.heads * self.dv)
+        return self.o(attended)
 
     def forward(self, x, ctx, binding: Binding, into=None):
         pages = ctx.groups[binding.group]
         key = self.rank + self.rot
         fused = ops.as_product(self.first(x))
         tokens = fused.rows
+        if self.expanded:
+            return self._forward_expanded(fused, ctx, binding)
         q_plain, q_wide = ops.latent_place(fused, ctx.positions, pages.slot_map if binding.writes else ctx.no_slots, self.inv_freq,
                                            self.down_norm, self.norm_eps, binding.cache, self.heads, self.plain, self.rot,
                                            self.rank, self.dtype, wide_values=self.wide_values, turn=self.turn,
