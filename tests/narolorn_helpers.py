@@ -70,11 +70,11 @@ CONFIG_Q = {        # a single residual, no loop, logits as they are; an attenti
     ],
 }
 CONFIG_R = {        # one stream (the three small tensors still act), a loop of a single layer; head sizes the matrix cores take
-    "architecture": "Narolorn", "vocab": 96, "width": 128, "norm": {"eps": 1e-5}, "streams": 1, "logit_softcap": 30.0,
+    "architecture": "Narolorn", "vocab": 96, "width": 128, "norm": {"eps": 1e-5}, "streams": 1, "logit_softcap": 25.0,
     "loop": {"start": 0, "stop": 1, "times": 2},
     "layers": [
-        {"type": "attention_2", "mixer": _attention_2(4, 2, 64, 0.125, chunk=24, rot=(20000.0, 32)), "mlp": _moe(4, 2, 32, 2.0, (32, 2.0))},
-        {"type": "attention", "mixer": _attention(2, 1, 64, 64, 0.125, softcap=20.0, q_temp=(0.5, 16)), "mlp": _moe(4, 1, 32, 2.0)},
+        {"type": "attention_2", "mixer": _attention_2(4, 2, 64, 0.12, chunk=24, rot=(30000.0, 32)), "mlp": _moe(4, 2, 32, 2.0, (32, 2.0))},
+        {"type": "attention", "mixer": _attention(2, 1, 64, 64, 0.13, softcap=20.0, q_temp=(0.7, 16)), "mlp": _moe(4, 1, 32, 2.0)},
         {"type": "latent_attention", "mixer": _latent(4, 32, 32, 64, 0.18, window=24), "mlp": _moe(6, 2, 16, 3.0, (64, 1.0))},
     ],
 }
